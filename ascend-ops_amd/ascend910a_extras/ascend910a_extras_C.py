@@ -1,0 +1,357 @@
+"""Binding layer between the Python API and the C-ABI kernel library.
+
+Takes the place of the reference's pybind module ``ascend910a_extras_C``
+(reference ``csrc/ffi/bind.cpp:53-61`` and ``csrc/ffi/ops.cpp:13-491``): an
+``ops`` namespace with one function per operator plus ``print_info``.  Each
+function repeats the reference's argument checks (same conditions, raised as
+``RuntimeError`` like ``TORCH_CHECK``), allocates the outputs, looks up the
+current HIP stream and calls ``libaops.so`` through ``ctypes`` with raw device
+pointers.  Nothing here synchronises or reads device data on the host.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import types
+
+import torch
+
+_LIB_NAME = "libaops.so"
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
+
+_vp = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_sz = ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/aops.h declaration by declaration.
+_SIGNATURES = {
+    "aops_version": (ctypes.c_int, []),
+    "aops_strerror": (ctypes.c_char_p, [ctypes.c_int]),
+    "aops_last_hip_error": (ctypes.c_int, []),
+    "aops_add_rms_norm_f16": (ctypes.c_int, [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _i64, _i64, _vp]),
+    "aops_swiglu_f16": (ctypes.c_int, [_vp, _vp, _i64, _i64, _vp]),
+    "aops_rope_neox_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "aops_reshape_and_cache_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "aops_grouped_matmul_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "aops_paged_attention_workspace": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64]),
+    "aops_paged_attention_f16": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
+    ),
+    "aops_device_info": (ctypes.c_int, [ctypes.c_int, ctypes.c_char_p, _sz]),
+}
+
+
+def _load_library() -> ctypes.CDLL:
+    if not os.path.exists(_LIB_PATH):
+        raise ImportError(
+            f"{_LIB_PATH} is missing: the HIP kernel library has not been built "
+            "(run `python ascend-ops_amd/build.py`). There is no fallback implementation."
+        )
+    lib = ctypes.CDLL(_LIB_PATH)
+    for name, (restype, argtypes) in _SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
+        fn.restype = restype
+        fn.argtypes = argtypes
+    return lib
+
+
+_lib = _load_library()
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def exported_symbols() -> list[str]:
+    return sorted(_SIGNATURES)
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _status(op: str, code: int) -> None:
+    if code != 0:
+        text = _lib.aops_strerror(code).decode()
+        extra = f" (hipError {_lib.aops_last_hip_error()})" if code == -3 else ""
+        raise RuntimeError(f"{op}: {text}{extra}")
+
+
+def _require_device(op: str, dtype_by_name: dict) -> None:
+    """dtype and device checks (the reference hard-codes ACL_FLOAT16/ACL_INT32/ACL_INT64)."""
+    device = None
+    for name, (t, dtype) in dtype_by_name.items():
+        _check(t.dtype == dtype, f"{op}: {name} must be {dtype}, got {t.dtype}")
+        _check(t.is_cuda, f"{op}: {name} must be on the GPU device, got {t.device}")
+        if device is None:
+            device = t.device
+        _check(t.device == device, f"{op}: all tensors must be on the same device")
+
+
+def _stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _ptr(t: torch.Tensor):
+    return t.data_ptr() if t.numel() > 0 else None
+
+
+def rope(q, k, position_ids, cos_cache, sin_cache):
+    """reference csrc/ffi/ops.cpp:13-108."""
+    _check(
+        q.dim() == 3 and k.dim() == 3 and position_ids.dim() == 1 and cos_cache.dim() == 2 and sin_cache.dim() == 2,
+        f"rope: input tensors must be 3D, 3D, 1D, 2D, and 2D, got {q.dim()}D, {k.dim()}D, "
+        f"{position_ids.dim()}D, {cos_cache.dim()}D, {sin_cache.dim()}D",
+    )
+    _check(
+        position_ids.size(0) == q.size(0),
+        f"rope: position_ids must have the same batch size as q, got {position_ids.size(0)} and {q.size(0)}",
+    )
+    _check(
+        q.is_contiguous() and k.is_contiguous() and position_ids.is_contiguous()
+        and cos_cache.is_contiguous() and sin_cache.is_contiguous(),
+        "rope: all input tensors must be contiguous",
+    )
+    bs, num_heads, head_dim = q.shape
+    _check(k.size(0) == bs and k.size(2) == head_dim, "rope: k must match q in batch size and head_dim")
+    _check(head_dim % 16 == 0, f"rope: head_dim must be a multiple of 16, got {head_dim}")
+    _check(
+        cos_cache.size(1) == head_dim // 2 and sin_cache.shape == cos_cache.shape,
+        f"rope: cos_cache and sin_cache must be [max_position, head_dim/2], got {tuple(cos_cache.shape)} "
+        f"and {tuple(sin_cache.shape)}",
+    )
+    _require_device(
+        "rope",
+        {
+            "q": (q, torch.float16), "k": (k, torch.float16), "position_ids": (position_ids, torch.int32),
+            "cos_cache": (cos_cache, torch.float16), "sin_cache": (sin_cache, torch.float16),
+        },
+    )
+    out_q = torch.empty_like(q)
+    out_k = torch.empty_like(k)
+    code = _lib.aops_rope_neox_f16(
+        _ptr(q), _ptr(k), _ptr(position_ids), _ptr(cos_cache), _ptr(sin_cache), _ptr(out_q), _ptr(out_k),
+        bs, num_heads, k.size(1), head_dim, _stream(q.device),
+    )
+    _status("rope", code)
+    return [out_q, out_k]
+
+
+def swiglu(x):
+    """reference csrc/ffi/ops.cpp:110-154."""
+    _check(x.dim() == 2, f"swiglu: input tensor must be 2D, got {x.dim()}D tensor")
+    _check(
+        x.size(-1) >= 64 and x.size(-1) % 64 == 0,
+        f"swiglu: last dimension must be a multiple of 64, got {x.size(-1)}",
+    )
+    _check(x.is_contiguous(), "swiglu: input tensor must be contiguous")
+    _require_device("swiglu", {"x": (x, torch.float16)})
+    y = torch.empty((x.size(0), x.size(1) // 2), dtype=x.dtype, device=x.device)
+    code = _lib.aops_swiglu_f16(_ptr(x), _ptr(y), x.size(0), x.size(1) // 2, _stream(x.device))
+    _status("swiglu", code)
+    return y
+
+
+def grouped_matmul(x, w, group_list):
+    """reference csrc/ffi/ops.cpp:157-233."""
+    _check(
+        x.dim() == 2 and w.dim() == 3 and group_list.dim() == 1,
+        "grouped_matmul: input tensors must be 2D and group_list must be 1D",
+    )
+    num_tokens, dim = x.shape
+    num_experts, inner_dim = w.size(0), w.size(2)
+    _check(
+        dim == w.size(1),
+        f"grouped_matmul: last dimension of x must match second dimension of w, got {dim} and {w.size(1)}",
+    )
+    _check(
+        x.is_contiguous() and group_list.is_contiguous(),
+        "grouped_matmul: x and group_list must be contiguous tensors",
+    )
+    _check(
+        w.stride(1) == 1 and w.stride(2) == dim,
+        f"grouped_matmul: w must be K-major order, got strides {tuple(w.stride())}",
+    )
+    _check(
+        w.size(1) % 64 == 0 and w.size(2) % 64 == 0,
+        f"grouped_matmul: second and third dimensions of w must be multiples of 64, got {w.size(1)} and {w.size(2)}",
+    )
+    _check(
+        num_experts <= 1 or w.stride(0) == dim * inner_dim,
+        f"grouped_matmul: experts of w must be densely packed, got strides {tuple(w.stride())}",
+    )
+    _check(
+        group_list.size(0) == num_experts,
+        f"grouped_matmul: group_list must have one entry per expert, got {group_list.size(0)} and {num_experts}",
+    )
+    _require_device(
+        "grouped_matmul",
+        {"x": (x, torch.float16), "w": (w, torch.float16), "group_list": (group_list, torch.int64)},
+    )
+    y = torch.empty((num_tokens, inner_dim), dtype=x.dtype, device=x.device)
+    code = _lib.aops_grouped_matmul_f16(
+        _ptr(x), _ptr(w), _ptr(group_list), _ptr(y), num_tokens, dim, num_experts, inner_dim, _stream(x.device)
+    )
+    _status("grouped_matmul", code)
+    return y
+
+
+def add_rms_norm(x, residual, weight, epsilon):
+    """reference csrc/ffi/ops.cpp:236-333."""
+    _check(
+        x.dim() == 2 and residual.dim() == 2 and weight.dim() == 1,
+        "add_rms_norm: x and residual must be 2D, weight must be 1D",
+    )
+    _check(
+        x.size(1) == weight.size(0),
+        f"add_rms_norm: last dimension of x must match weight size, got {x.size(1)} and {weight.size(0)}",
+    )
+    _check(
+        x.size(0) == residual.size(0) and x.size(1) == residual.size(1),
+        f"add_rms_norm: x and residual must have the same shape, got {tuple(x.shape)} and {tuple(residual.shape)}",
+    )
+    _check(
+        x.is_contiguous() and residual.is_contiguous() and weight.is_contiguous(),
+        "add_rms_norm: all input tensors must be contiguous",
+    )
+    _check(x.size(1) % 64 == 0, f"add_rms_norm: last dimension must be a multiple of 64, got {x.size(1)}")
+    _require_device(
+        "add_rms_norm",
+        {"x": (x, torch.float16), "residual": (residual, torch.float16), "weight": (weight, torch.float16)},
+    )
+    y = torch.empty_like(x)
+    residual_output = torch.empty_like(x)
+    code = _lib.aops_add_rms_norm_f16(
+        _ptr(x), _ptr(residual), _ptr(weight), float(epsilon), _ptr(y), _ptr(residual_output),
+        x.size(0), x.size(1), _stream(x.device),
+    )
+    _status("add_rms_norm", code)
+    return y, residual_output
+
+
+def reshape_and_cache(key, value, key_cache, value_cache, slot_indices):
+    """reference csrc/ffi/ops.cpp:336-405; an empty ``value``/``value_cache`` means "not given"."""
+    _check(
+        key.dim() == 3 and key_cache.dim() == 4 and slot_indices.dim() == 1,
+        "reshape_and_cache: key must be 3D, key_cache must be 4D, slot_indices must be 1D",
+    )
+    _check(
+        key.is_contiguous() and key_cache.is_contiguous() and slot_indices.is_contiguous(),
+        "reshape_and_cache: key, key_cache, slot_indices must be contiguous tensors",
+    )
+    if value.numel() > 0:
+        _check(value.dim() == 3 and value.is_contiguous(), "reshape_and_cache: value must be 3D and contiguous if not None")
+    if value_cache.numel() > 0:
+        _check(
+            value_cache.dim() == 4 and value_cache.is_contiguous(),
+            "reshape_and_cache: value_cache must be 4D and contiguous if not None",
+        )
+    num_tokens, num_kv_heads, head_size = key.shape
+    num_blocks, nh16, block_size, chunk = key_cache.shape
+    # reference csrc/opdev/op_host/reshape_and_cache_ex.cpp:31-36
+    _check(
+        slot_indices.size(0) == num_tokens,
+        f"reshape_and_cache: slot_indices length must equal num_tokens, got {slot_indices.size(0)} and {num_tokens}",
+    )
+    _check(
+        chunk == 16 and nh16 * 16 == num_kv_heads * head_size,
+        f"reshape_and_cache: key_cache must be [num_blocks, num_kv_heads*head_size/16, block_size, 16], "
+        f"got {tuple(key_cache.shape)} for key {tuple(key.shape)}",
+    )
+    tensors = {
+        "key": (key, torch.float16), "key_cache": (key_cache, torch.float16),
+        "slot_indices": (slot_indices, torch.int32),
+    }
+    with_value = value.numel() > 0 and value_cache.numel() > 0
+    if with_value:
+        _check(value.shape == key.shape, "reshape_and_cache: value must have the shape of key")
+        _check(value_cache.shape == key_cache.shape, "reshape_and_cache: value_cache must have the shape of key_cache")
+        tensors["value"] = (value, torch.float16)
+        tensors["value_cache"] = (value_cache, torch.float16)
+    _require_device("reshape_and_cache", tensors)
+    code = _lib.aops_reshape_and_cache_f16(
+        _ptr(key), _ptr(value) if with_value else None, _ptr(key_cache),
+        _ptr(value_cache) if with_value else None, _ptr(slot_indices),
+        num_tokens, num_kv_heads * head_size, num_blocks, block_size, _stream(key.device),
+    )
+    _status("reshape_and_cache", code)
+    return None
+
+
+def paged_attention(q, key_cache, value_cache, block_tables, context_lens):
+    """reference csrc/ffi/ops.cpp:408-482 (which performs no checks; the shapes it assumes are
+    enforced here)."""
+    _check(
+        q.dim() == 3 and key_cache.dim() == 4 and value_cache.dim() == 4
+        and block_tables.dim() == 2 and context_lens.dim() == 1,
+        "paged_attention: q must be 3D, key_cache and value_cache 4D, block_tables 2D, context_lens 1D",
+    )
+    _check(
+        q.is_contiguous() and key_cache.is_contiguous() and value_cache.is_contiguous()
+        and block_tables.is_contiguous() and context_lens.is_contiguous(),
+        "paged_attention: all input tensors must be contiguous",
+    )
+    bs, num_heads, head_dim = q.shape
+    num_blocks, nh16, block_size, chunk = key_cache.shape
+    _check(chunk == 16, f"paged_attention: last dimension of the caches must be 16, got {chunk}")
+    _check(value_cache.shape == key_cache.shape, "paged_attention: key_cache and value_cache must have the same shape")
+    _check(
+        head_dim > 0 and (nh16 * 16) % head_dim == 0 and nh16 * 16 >= head_dim,
+        f"paged_attention: cache rows ({nh16 * 16} halfs) must hold whole heads of {head_dim}",
+    )
+    num_kv_heads = nh16 * 16 // head_dim
+    _check(
+        num_heads % num_kv_heads == 0,
+        f"paged_attention: num_heads ({num_heads}) must be a multiple of num_kv_heads ({num_kv_heads})",
+    )
+    _check(
+        block_tables.size(0) == bs and context_lens.size(0) == bs,
+        "paged_attention: block_tables and context_lens must have one row per sequence",
+    )
+    _require_device(
+        "paged_attention",
+        {
+            "q": (q, torch.float16), "key_cache": (key_cache, torch.float16),
+            "value_cache": (value_cache, torch.float16), "block_tables": (block_tables, torch.int32),
+            "context_lens": (context_lens, torch.int32),
+        },
+    )
+    max_blocks = block_tables.size(1)
+    o = torch.empty_like(q)
+    if bs == 0:
+        return o
+    ws_bytes = _lib.aops_paged_attention_workspace(bs, num_heads, num_kv_heads, head_dim, block_size, max_blocks)
+    _check(
+        ws_bytes > 0,
+        f"paged_attention: unsupported shape (head_dim={head_dim}, block_size={block_size}, "
+        f"group={num_heads // num_kv_heads}); head_dim must be 128, block_size a multiple of 32 and "
+        "num_heads/num_kv_heads one of 1, 2, 4, 8",
+    )
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    code = _lib.aops_paged_attention_f16(
+        _ptr(q), _ptr(key_cache), _ptr(value_cache), _ptr(block_tables), _ptr(context_lens), _ptr(o),
+        _ptr(workspace), ws_bytes, bs, num_heads, num_kv_heads, head_dim, block_size, max_blocks,
+        num_blocks, _stream(q.device),
+    )
+    _status("paged_attention", code)
+    return o
+
+
+def print_info(device_id: int) -> None:
+    """reference csrc/ffi/bind.cpp:26-51."""
+    buf = ctypes.create_string_buffer(1024)
+    n = _lib.aops_device_info(int(device_id), buf, len(buf))
+    _status("print_info", n if n < 0 else 0)
+    print(buf.value.decode(), end="")
+
+
+ops = types.SimpleNamespace(
+    rope=rope,
+    swiglu=swiglu,
+    grouped_matmul=grouped_matmul,
+    add_rms_norm=add_rms_norm,
+    reshape_and_cache=reshape_and_cache,
+    paged_attention=paged_attention,
+)

@@ -1,0 +1,101 @@
+"""Builds libaops.so (the C-ABI library of gfx950 HIP kernels) in-tree with hipcc.
+
+Usage: ``python build.py [--force]`` or ``from build import build_library``.
+The library is written next to the Python package that loads it
+(``ascend910a_extras/libaops.so``).
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+HERE = Path(__file__).resolve().parent
+CSRC = HERE / "csrc"
+INCLUDE = HERE.parent / "include"
+OUT_DIR = HERE / "ascend910a_extras"
+LIB_NAME = "libaops.so"
+ARCH = "gfx950"
+
+SOURCES = [
+    "aops_api.hip",
+    "add_rms_norm.hip",
+    "swiglu.hip",
+    "rope.hip",
+    "reshape_and_cache.hip",
+    "paged_attention.hip",
+    "grouped_matmul.hip",
+]
+
+# -packed-fp32-ops: keep the compiler from forming packed-fp32 VALU instructions.
+HIPCC_FLAGS = [
+    f"--offload-arch={ARCH}",
+    "-O3",
+    "-fPIC",
+    "-std=c++17",
+    "-fno-gpu-rdc",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    f"-I{INCLUDE}",
+    f"-I{CSRC}",
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found: the HIP kernels cannot be built")
+    return exe
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(
+        line for line in proc.stdout.splitlines() if "is not a recognized feature" not in line
+    )
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(map(str, cmd)), out))
+    return out
+
+
+def library_path() -> Path:
+    return OUT_DIR / LIB_NAME
+
+
+def build_library(force: bool = True, verbose: bool = False) -> Path:
+    """Compiles every HIP source for gfx950 and links the shared library."""
+    hipcc = _hipcc()
+    obj_dir = HERE / "build" / "obj"
+    obj_dir.mkdir(parents=True, exist_ok=True)
+    headers = list(CSRC.glob("*.h")) + list(INCLUDE.glob("*.h"))
+    newest_header = max(h.stat().st_mtime for h in headers)
+
+    def compile_one(name: str) -> Path:
+        src = CSRC / name
+        obj = obj_dir / (name + ".o")
+        stale = (
+            force
+            or not obj.exists()
+            or obj.stat().st_mtime < max(src.stat().st_mtime, newest_header)
+        )
+        if stale:
+            out = _run([hipcc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)])
+            if verbose and out.strip():
+                print(out)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+        objs = list(pool.map(compile_one, SOURCES))
+    lib = library_path()
+    tmp = lib.with_suffix(".so.tmp")
+    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)])
+    os.replace(tmp, lib)
+    return lib
+
+
+if __name__ == "__main__":
+    path = build_library(force="--force" in sys.argv, verbose=True)
+    print(path)

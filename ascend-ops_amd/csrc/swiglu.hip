@@ -1,0 +1,64 @@
+// SwiGLU: y[t, j] = silu(x[t, j]) * x[t, d + j], fp16 in/out, fp32 math.
+// Pure streaming op: 6*d bytes per row (4d read, 2d written), 128-bit accesses.
+// Semantics: reference csrc/opdev/op_kernel/swi_glu_ex.cpp:54-56, benchmark/test_swiglu.py:6-12.
+#include "aops_common.h"
+
+namespace aops {
+
+__device__ __forceinline__ f16x8 silu_mul(f16x8 g, f16x8 u) {
+  f16x8 o;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float a = (float)g[j];
+    const float b = (float)u[j];
+    // a * sigmoid(a) = a / (1 + 2^(-a*log2 e))
+    const float e = __builtin_amdgcn_exp2f(-1.4426950408889634f * a);
+    o[j] = (f16)(a * b * __builtin_amdgcn_rcpf(1.0f + e));
+  }
+  return o;
+}
+
+template <int UNROLL>
+__global__ __launch_bounds__(256) void swiglu_kernel(const f16* __restrict__ x,
+                                                     f16* __restrict__ y, uint32_t total_vec,
+                                                     uint32_t vec_per_row, int64_t d) {
+  const uint32_t base = (blockIdx.x * UNROLL) * 256u + threadIdx.x;
+  f16x8 g[UNROLL], u[UNROLL];
+  uint32_t row[UNROLL], col[UNROLL];
+#pragma unroll
+  for (int i = 0; i < UNROLL; ++i) {
+    const uint32_t v = base + i * 256u;
+    if (v < total_vec) {
+      row[i] = v / vec_per_row;
+      col[i] = v - row[i] * vec_per_row;
+      const f16* p = x + (int64_t)row[i] * (2 * d) + (int64_t)col[i] * 8;
+      g[i] = ld128_stream(p);
+      u[i] = ld128_stream(p + d);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < UNROLL; ++i) {
+    const uint32_t v = base + i * 256u;
+    if (v < total_vec)
+      st128_stream(y + (int64_t)row[i] * d + (int64_t)col[i] * 8, silu_mul(g[i], u[i]));
+  }
+}
+
+}  // namespace aops
+
+extern "C" int aops_swiglu_f16(const void* x, void* y, int64_t num_tokens, int64_t d,
+                               void* stream) {
+  using namespace aops;
+  if (num_tokens < 0 || d <= 0 || d % 8 != 0) return AOPS_ERR_INVALID_ARGUMENT;
+  if (num_tokens == 0) return AOPS_OK;
+  if (!x || !y) return AOPS_ERR_INVALID_ARGUMENT;
+  const int64_t vec_per_row = d / 8;
+  const int64_t total = num_tokens * vec_per_row;
+  if (total >= ((int64_t)1 << 32) - 4096) return AOPS_ERR_INVALID_ARGUMENT;
+  constexpr int kUnroll = 2;
+  const unsigned grid = (unsigned)((total + 256 * kUnroll - 1) / (256 * kUnroll));
+  swiglu_kernel<kUnroll><<<grid, 256, 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<const f16*>(x), static_cast<f16*>(y), (uint32_t)total, (uint32_t)vec_per_row,
+      d);
+  return record_launch_status(hipGetLastError());
+}

@@ -1,0 +1,138 @@
+/*
+ * aops.h -- C ABI of the MI355X (gfx950) implementation of the
+ * ascend910a_extras operator set.
+ *
+ * Every entry point takes raw DEVICE pointers and sizes, enqueues its kernels
+ * on the HIP stream it is given (hipStream_t passed as void*; NULL = the
+ * default stream) and returns without synchronising.  No entry point reads
+ * device data on the host, so all of them can be captured into a HIP graph.
+ * Return value: AOPS_OK (0) or a negative AOPS_ERR_* code; nothing is thrown
+ * across this boundary.  All fp tensors are IEEE binary16 ("f16"), densely
+ * packed and row-major in the shapes stated.
+ *
+ * Each declaration names the reference interface it replaces: the two-phase
+ * aclnn*GetWorkspaceSize / aclnn* pair that csrc/ffi/ops.cpp of the reference
+ * calls for that operator.
+ */
+#ifndef AOPS_H_
+#define AOPS_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AOPS_OK 0
+#define AOPS_ERR_INVALID_ARGUMENT (-1) /* null pointer, negative size, size the kernels do not support */
+#define AOPS_ERR_WORKSPACE (-2)        /* workspace missing or too small */
+#define AOPS_ERR_LAUNCH (-3)           /* HIP reported an error at launch; see aops_last_hip_error() */
+
+/* Library version (major*10000 + minor*100 + patch). */
+int aops_version(void);
+
+/* Text for an AOPS_ERR_* code (static storage). */
+const char* aops_strerror(int code);
+
+/* hipError_t of the last failed launch on the calling thread (0 if none). */
+int aops_last_hip_error(void);
+
+/*
+ * Fused residual add + RMSNorm.
+ *   t = x + residual (fp32); residual_out = f16(t);
+ *   y = f16(t * rsqrt(mean(t^2) + eps) * weight)
+ * x, residual, y, residual_out: [num_tokens, hidden]; weight: [hidden].
+ * hidden must be a multiple of 8.  y/residual_out must not alias the inputs.
+ * Replaces aclnnAddRMSNormExGetWorkspaceSize + aclnnAddRMSNormEx
+ * (reference csrc/ffi/ops.cpp:303-310).
+ */
+int aops_add_rms_norm_f16(const void* x, const void* residual, const void* weight, float epsilon,
+                          void* y, void* residual_out, int64_t num_tokens, int64_t hidden,
+                          void* stream);
+
+/*
+ * SwiGLU: y[t, j] = f16(silu(x[t, j]) * x[t, d + j]), x: [num_tokens, 2*d], y: [num_tokens, d].
+ * d must be a multiple of 8.
+ * Replaces aclnnSwiGluExGetWorkspaceSize + aclnnSwiGluEx (reference csrc/ffi/ops.cpp:138-145).
+ */
+int aops_swiglu_f16(const void* x, void* y, int64_t num_tokens, int64_t d, void* stream);
+
+/*
+ * Neox (rotate-half) rotary embedding on q and k.
+ * q: [bs, num_heads, head_dim], k: [bs, num_kv_heads, head_dim], position_ids: int32 [bs],
+ * cos_cache, sin_cache: [max_position, head_dim/2]; out_q/out_k like q/k.
+ * head_dim must be a multiple of 16.  position_ids are not range-checked.
+ * Replaces aclnnRopeExGetWorkspaceSize + aclnnRopeEx (reference csrc/ffi/ops.cpp:76-83).
+ */
+int aops_rope_neox_f16(const void* q, const void* k, const int32_t* position_ids,
+                       const void* cos_cache, const void* sin_cache, void* out_q, void* out_k,
+                       int64_t bs, int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                       void* stream);
+
+/*
+ * Scatter of new K (and optionally V) rows into the paged cache.
+ * key, value: [num_tokens, row_elems] with row_elems = num_kv_heads*head_dim (multiple of 16);
+ * key_cache, value_cache: [num_blocks, row_elems/16, block_size, 16];
+ * slot_indices: int32 [num_tokens].  For token t with s = slot_indices[t]:
+ *   cache[s / block_size, c, s % block_size, 0:16] = row[t, 16c : 16c+16]   for every c.
+ * Slots outside [0, num_blocks*block_size) are skipped.  value and value_cache may both be
+ * NULL (key only); if only one of them is NULL the value side is skipped.
+ * Replaces aclnnReshapeAndCacheExGetWorkspaceSize + aclnnReshapeAndCacheEx
+ * (reference csrc/ffi/ops.cpp:387-396).
+ */
+int aops_reshape_and_cache_f16(const void* key, const void* value, void* key_cache,
+                               void* value_cache, const int32_t* slot_indices, int64_t num_tokens,
+                               int64_t row_elems, int64_t num_blocks, int64_t block_size,
+                               void* stream);
+
+/*
+ * Grouped (per-expert) matmul over expert-sorted rows.
+ * x: [rows, k]; w: [num_experts, n, k] (each expert's weight stored N-major, K contiguous --
+ * the logical [E, K, N] tensor with stride(1)==1, stride(2)==K); group_list: int64
+ * [num_experts] cumulative row ends, read on the device; y: [rows, n].
+ *   y[group_list[e-1] : group_list[e], :] = f16( x[...] (fp32 accumulate) @ w[e]^T )
+ * Rows at or past group_list[num_experts-1] are not written.  k and n must be multiples of 64.
+ * Replaces aclnnGroupedMatMulExGetWorkspaceSize + aclnnGroupedMatMulEx
+ * (reference csrc/ffi/ops.cpp:211-218).
+ */
+int aops_grouped_matmul_f16(const void* x, const void* w, const int64_t* group_list, void* y,
+                            int64_t rows, int64_t k, int64_t num_experts, int64_t n,
+                            void* stream);
+
+/*
+ * Paged-attention decode (one query token per sequence).
+ * q, o: [bs, num_heads, head_dim]; key_cache, value_cache:
+ * [num_blocks, num_kv_heads*head_dim/16, block_size, 16]; block_tables: int32
+ * [bs, max_blocks_per_seq]; context_lens: int32 [bs] (read on the device).
+ *   o[b,h] = softmax_j( q[b,h] . K[j,g] / sqrt(head_dim) ) . V[j,g],  g = h / (num_heads/num_kv_heads)
+ * The kernels split every sequence into fixed-size chunks of the KV cache and keep partial
+ * results in `workspace`; aops_paged_attention_workspace() returns the bytes needed (the
+ * counterpart of the reference's GetWorkspaceSize phase).  A sequence with context_len <= 0
+ * gets zeros.  Block-table entries are not range-checked.
+ * Replaces aclnnPagedAttentionExGetWorkspaceSize + aclnnPagedAttentionEx
+ * (reference csrc/ffi/ops.cpp:454-461).
+ */
+size_t aops_paged_attention_workspace(int64_t bs, int64_t num_heads, int64_t num_kv_heads,
+                                      int64_t head_dim, int64_t block_size,
+                                      int64_t max_blocks_per_seq);
+
+int aops_paged_attention_f16(const void* q, const void* key_cache, const void* value_cache,
+                             const int32_t* block_tables, const int32_t* context_lens, void* o,
+                             void* workspace, size_t workspace_bytes, int64_t bs,
+                             int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                             int64_t block_size, int64_t max_blocks_per_seq, int64_t num_blocks,
+                             void* stream);
+
+/*
+ * Device summary (CU count, LDS, L2, memory size, clocks) written as text into buf
+ * (at most buf_len bytes including the terminator).  Returns the length written or a
+ * negative code.  Replaces print_info (reference csrc/ffi/bind.cpp:26-51).
+ */
+int aops_device_info(int device, char* buf, size_t buf_len);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* AOPS_H_ */

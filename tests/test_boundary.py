@@ -1,0 +1,135 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports every symbol
+include/aops.h declares, and the Python layer rejects what the reference's ffi rejects
+(reference csrc/ffi/ops.cpp TORCH_CHECKs) with RuntimeError."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "aops.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(aops_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    import ascend910a_extras.ascend910a_extras_C as C
+
+    declared = _declared_symbols()
+    assert len(declared) >= 11
+    lib = ctypes.CDLL(C.library_path())
+    for name in declared:
+        assert hasattr(lib, name), f"libaops.so lacks {name}"
+    # the ctypes signature table covers exactly the declared functions
+    assert C.exported_symbols() == declared
+    assert C._lib.aops_version() >= 100
+    assert C._lib.aops_strerror(0) == b"success"
+    assert b"workspace" in C._lib.aops_strerror(-2)
+
+
+def test_api_surface_matches_reference_ops_py():
+    import inspect
+
+    import ascend910a_extras.ops as ops
+
+    want = {
+        "rope": ["q", "k", "position_ids", "cos_cache", "sin_cache"],
+        "swiglu": ["x"],
+        "grouped_matmul": ["x", "w", "group_list"],
+        "add_rms_norm": ["x", "residual", "weight", "epsilon"],
+        "reshape_and_cache": ["key", "value", "key_cache", "value_cache", "slot_indices"],
+        "paged_attention": ["q", "key_cache", "value_cache", "block_tables", "context_lens"],
+        "print_info": [],
+    }
+    for name, params in want.items():
+        assert list(inspect.signature(getattr(ops, name)).parameters) == params
+    assert inspect.signature(ops.add_rms_norm).parameters["epsilon"].default == 1e-5
+
+
+def test_workspace_query_without_gpu():
+    import ascend910a_extras.ascend910a_extras_C as C
+
+    # config 5 shape: 64 x 32 heads, 8 kv heads, D=128, P=128, 32 pages -> 8 chunks of 512
+    n = C._lib.aops_paged_attention_workspace(64, 32, 8, 128, 128, 32)
+    assert n == 64 * 32 * 8 * 130 * 4
+    assert C._lib.aops_paged_attention_workspace(64, 32, 8, 96, 128, 32) == 0  # unsupported head_dim
+    assert C._lib.aops_paged_attention_workspace(64, 32, 8, 128, 24, 32) == 0  # unsupported page size
+
+
+def test_c_abi_rejects_bad_sizes_without_touching_the_gpu():
+    import ascend910a_extras.ascend910a_extras_C as C
+
+    lib = C._lib
+    assert lib.aops_swiglu_f16(None, None, 4, 12, None) == -1  # d % 8
+    assert lib.aops_swiglu_f16(None, None, 4, 64, None) == -1  # null pointers
+    assert lib.aops_swiglu_f16(None, None, 0, 64, None) == 0   # empty input is a no-op
+    assert lib.aops_add_rms_norm_f16(None, None, None, 1e-6, None, None, 4, 100, None) == -1
+    assert lib.aops_add_rms_norm_f16(None, None, None, 1e-6, None, None, 0, 128, None) == 0
+    assert lib.aops_rope_neox_f16(None, None, None, None, None, None, None, 2, 4, 2, 24, None) == -1
+    assert lib.aops_reshape_and_cache_f16(None, None, None, None, None, 4, 1000, 8, 16, None) == -1
+    assert lib.aops_reshape_and_cache_f16(None, None, None, None, None, 0, 1024, 8, 16, None) == 0
+    assert lib.aops_grouped_matmul_f16(None, None, None, None, 16, 100, 2, 64, None) == -1
+    assert lib.aops_grouped_matmul_f16(None, None, None, None, 0, 64, 2, 64, None) == 0
+    assert lib.aops_paged_attention_f16(None, None, None, None, None, None, None, 0, 2, 8, 2, 64, 128, 4, 16, None) == -1
+
+
+H = torch.float16
+
+
+def _raises(fn, *args, match=None):
+    with pytest.raises(RuntimeError, match=match):
+        fn(*args)
+
+
+def test_argument_checks_follow_the_reference(ops):
+    # swiglu: 2-D, last dim >= 64 and % 64, contiguous (reference csrc/ffi/ops.cpp:111-116)
+    _raises(ops.swiglu, torch.zeros(2, 3, 64, dtype=H), match="2D")
+    _raises(ops.swiglu, torch.zeros(4, 96, dtype=H), match="multiple of 64")
+    _raises(ops.swiglu, torch.zeros(128, 4, dtype=H).t(), match="contiguous")
+    # add_rms_norm (reference csrc/ffi/ops.cpp:237-246)
+    _raises(ops.add_rms_norm, torch.zeros(4, 64, dtype=H), torch.zeros(4, 64, dtype=H), torch.zeros(1, 64, dtype=H), 1e-6, match="1D")
+    _raises(ops.add_rms_norm, torch.zeros(4, 64, dtype=H), torch.zeros(4, 64, dtype=H), torch.zeros(128, dtype=H), 1e-6, match="weight size")
+    _raises(ops.add_rms_norm, torch.zeros(4, 64, dtype=H), torch.zeros(5, 64, dtype=H), torch.zeros(64, dtype=H), 1e-6, match="same shape")
+    _raises(ops.add_rms_norm, torch.zeros(4, 96, dtype=H), torch.zeros(4, 96, dtype=H), torch.zeros(96, dtype=H), 1e-6, match="multiple of 64")
+    # grouped_matmul (reference csrc/ffi/ops.cpp:158-174)
+    x = torch.zeros(8, 64, dtype=H)
+    w_ok = torch.zeros(2, 128, 64, dtype=H).transpose(1, 2)
+    gl = torch.tensor([4, 8])
+    _raises(ops.grouped_matmul, x, torch.zeros(2, 64, 128, dtype=H), gl, match="K-major")
+    _raises(ops.grouped_matmul, torch.zeros(8, 128, dtype=H), w_ok, gl, match="must match")
+    _raises(ops.grouped_matmul, x, w_ok[0], gl, match="2D")
+    _raises(ops.grouped_matmul, torch.zeros(8, 96, dtype=H), torch.zeros(2, 128, 96, dtype=H).transpose(1, 2), gl, match="multiples of 64")
+    # rope (reference csrc/ffi/ops.cpp:14-19)
+    q = torch.zeros(2, 4, 64, dtype=H); k = torch.zeros(2, 2, 64, dtype=H)
+    cs = torch.zeros(16, 32, dtype=H)
+    _raises(ops.rope, q, k, torch.zeros(3, dtype=torch.int32), cs, cs, match="batch size")
+    _raises(ops.rope, q[0], k, torch.zeros(2, dtype=torch.int32), cs, cs, match="3D")
+    _raises(ops.rope, q.transpose(0, 1), k, torch.zeros(4, dtype=torch.int32), cs, cs, match="contiguous")
+    # reshape_and_cache (reference csrc/ffi/ops.cpp:337-347, op_host/reshape_and_cache_ex.cpp:31-36)
+    key = torch.zeros(4, 2, 64, dtype=H); cache = torch.zeros(3, 8, 16, 16, dtype=H)
+    slots = torch.zeros(4, dtype=torch.int32)
+    _raises(ops.reshape_and_cache, key[0], None, cache, None, slots, match="3D")
+    _raises(ops.reshape_and_cache, key, None, cache, None, slots[:3], match="num_tokens")
+    _raises(ops.reshape_and_cache, key, key[0], cache, cache, slots, match="value must be 3D")
+    _raises(ops.reshape_and_cache, key, None, torch.zeros(3, 4, 16, 16, dtype=H), None, slots, match="key_cache must be")
+    # paged_attention: shapes the reference assumes silently
+    _raises(ops.paged_attention, torch.zeros(2, 8, 128, dtype=H), torch.zeros(4, 16, 128, 8, dtype=H),
+            torch.zeros(4, 16, 128, 8, dtype=H), torch.zeros(2, 2, dtype=torch.int32), torch.zeros(2, dtype=torch.int32), match="16")
+    # valid arguments on the CPU are refused: there is no CPU implementation to fall back to
+    _raises(ops.swiglu, torch.zeros(4, 128, dtype=H), match="GPU device")
+    _raises(ops.add_rms_norm, torch.zeros(4, 64, dtype=H), torch.zeros(4, 64, dtype=H), torch.zeros(64, dtype=H), 1e-6, match="GPU device")
+    _raises(ops.swiglu, torch.zeros(4, 128, dtype=torch.float32), match="float16")
+
+
+def test_product_package_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "ascend-ops_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, f"{f} mentions the oracle"

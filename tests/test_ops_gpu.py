@@ -1,0 +1,349 @@
+"""GPU parity tests: every operator, called through the Python API (and so through the C ABI
+of libaops.so), against the CPU oracle on the same seeded inputs.
+
+Bars (from the project's statement of parity): reshape_and_cache bit-exact; fp16 operators
+within rtol = atol = 1e-2 of the fp32 oracle; grouped_matmul within rtol = atol = 2e-2."""
+import math
+
+import pytest
+import torch
+
+import oracle.ops_ref as R
+
+pytestmark = pytest.mark.gpu
+H = torch.float16
+TOL = dict(rtol=1e-2, atol=1e-2)
+GMM_TOL = dict(rtol=2e-2, atol=2e-2)
+
+
+def _gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+# ----------------------------------------------------------------------------- add_rms_norm
+@pytest.mark.parametrize(
+    "T,Hd,eps",
+    [(128, 4096, 1e-6), (1024, 1024, 1e-6), (1, 64, 1e-5), (7, 192, 1e-6), (3, 8192, 1e-6),
+     (2, 16384, 1e-6), (2, 65536, 1e-6), (2, 65536 + 64, 1e-6), (4096, 4096, 1e-6), (0, 128, 1e-6)],
+)
+def test_add_rms_norm(ops, dev, T, Hd, eps):
+    g = _gen(0)
+    x = torch.randn(T, Hd, generator=g).half()
+    r = torch.randn(T, Hd, generator=g).half()
+    w = (1 + 0.1 * torch.randn(Hd, generator=g)).half()
+    y_ref, res_ref = R.add_rms_norm_ref(x, r, w, eps)
+    xd, rd = x.to(dev), r.to(dev)
+    y, res = ops.add_rms_norm(xd, rd, w.to(dev), eps)
+    torch.cuda.synchronize()
+    assert y.shape == (T, Hd) and y.dtype == H
+    assert torch.equal(res.cpu(), res_ref)  # fp16 sum is exactly determined
+    torch.testing.assert_close(y.cpu().float(), y_ref.float(), **TOL)
+    assert torch.equal(xd.cpu(), x) and torch.equal(rd.cpu(), r)  # inputs untouched
+
+
+def test_add_rms_norm_default_epsilon_and_reference_script_shape(ops, dev):
+    # benchmark/test_add_rms_norm.py:14-22: T=1024, dim=1024, weight ~ N(0,1); its tolerance is 1e-3
+    g = _gen(0)
+    x = torch.randn(1024, 1024, generator=g).half()
+    r = torch.randn(1024, 1024, generator=g).half()
+    w = torch.randn(1024, generator=g).half()
+    y_ref, res_ref = R.add_rms_norm_ref(x, r, w, 1e-6)
+    y, res = ops.add_rms_norm(x.to(dev), r.to(dev), w.to(dev), 1e-6)
+    torch.testing.assert_close(y.cpu(), y_ref, atol=4e-3, rtol=4e-3)
+    torch.testing.assert_close(res.cpu(), res_ref, atol=1e-3, rtol=1e-3)
+    y5, _ = ops.add_rms_norm(x.to(dev), r.to(dev), w.to(dev))  # epsilon defaults to 1e-5
+    y5_ref, _ = R.add_rms_norm_ref(x, r, w, 1e-5)
+    torch.testing.assert_close(y5.cpu().float(), y5_ref.float(), **TOL)
+
+
+# ----------------------------------------------------------------------------- swiglu
+@pytest.mark.parametrize("T,d", [(256, 14336), (2048, 192), (32768, 768), (1, 32), (5, 96), (3, 4000), (0, 64)])
+def test_swiglu(ops, dev, T, d):
+    x = torch.randn(T, 2 * d, generator=_gen(0)).half()
+    if T > 0:
+        x[0, :8] = torch.tensor([0.0, -0.0, 20.0, -20.0, 65504.0, -65504.0, 1e-4, -1e-4]).half()
+    y = ops.swiglu(x.to(dev))
+    assert y.shape == (T, d)
+    torch.testing.assert_close(y.cpu().float(), R.swiglu_ref(x).float(), **TOL)
+
+
+# ----------------------------------------------------------------------------- rope
+@pytest.mark.parametrize("B,Hq,Hkv,D,max_pos", [(64, 32, 8, 128, 4096), (4, 32, 8, 128, 40960), (1, 1, 1, 16, 8), (3, 5, 5, 64, 100), (2, 16, 2, 256, 64)])
+def test_rope(ops, dev, B, Hq, Hkv, D, max_pos):
+    g = _gen(0)
+    q = torch.randn(B, Hq, D, generator=g).half()
+    k = torch.randn(B, Hkv, D, generator=g).half()
+    cos, sin = R.build_cos_sin_cache(max_pos, D, theta=1e6)
+    pos = torch.randint(0, max_pos, (B,), generator=g, dtype=torch.int32)
+    pos[0] = 0
+    pos[-1] = max_pos - 1
+    out = ops.rope(q.to(dev), k.to(dev), pos.to(dev), cos.to(dev), sin.to(dev))
+    assert isinstance(out, (list, tuple)) and len(out) == 2
+    rq, rk = R.rope_ref(q, k, pos, cos, sin)
+    torch.testing.assert_close(out[0].cpu().float(), rq.float(), **TOL)
+    torch.testing.assert_close(out[1].cpu().float(), rk.float(), **TOL)
+    if B > 1:
+        assert torch.equal(out[0][0].cpu(), q[0])  # position 0 is the identity, exactly
+    # native-fp16 evaluation of the reference formula also agrees within tolerance
+    nq, _ = R.rope_ref(q, k, pos, cos, sin, compute_dtype=H)
+    torch.testing.assert_close(out[0].cpu().float(), nq.float(), **TOL)
+
+
+# ----------------------------------------------------------------------------- reshape_and_cache
+def test_reshape_and_cache_reference_known_answer(ops, dev):
+    """benchmark/test_reshape_and_cache.py:29-84 on the GPU, both of its cases, bit-exact."""
+    torch.manual_seed(42)
+    slots = torch.tensor([6, 134, 212, 290], dtype=torch.int32)
+    key = torch.randn(4, 8, 128, dtype=H)
+    value = torch.randn(4, 8, 128, dtype=H)
+    kc_ref = torch.zeros(583, 64, 128, 16, dtype=H); vc_ref = torch.zeros_like(kc_ref)
+    R.reshape_and_cache_ref(key, kc_ref, slots, value, vc_ref)
+    kc = torch.zeros_like(kc_ref, device=dev); vc = torch.zeros_like(kc_ref, device=dev)
+    assert ops.reshape_and_cache(key.to(dev), value.to(dev), kc, vc, slots.to(dev)) is None
+    assert torch.equal(kc.cpu(), kc_ref) and torch.equal(vc.cpu(), vc_ref)
+    key2 = torch.randn(4, 8, 128, dtype=H)
+    kc2_ref = torch.zeros_like(kc_ref)
+    R.reshape_and_cache_ref(key2, kc2_ref, slots)
+    kc2 = torch.zeros_like(kc_ref, device=dev); vc2 = torch.zeros_like(kc_ref, device=dev)
+    ops.reshape_and_cache(key2.to(dev), None, kc2, None, slots.to(dev))
+    assert torch.equal(kc2.cpu(), kc2_ref)
+    assert torch.count_nonzero(vc2) == 0
+
+
+@pytest.mark.parametrize("T,Hkv,D,NB,P", [(2048, 8, 128, 1024, 128), (64, 8, 128, 40, 128), (17, 2, 64, 9, 16), (5, 1, 16, 3, 7), (0, 8, 128, 4, 128)])
+def test_reshape_and_cache_bit_exact(ops, dev, T, Hkv, D, NB, P):
+    g = _gen(0)
+    key = torch.randn(T, Hkv, D, generator=g).half()
+    value = torch.randn(T, Hkv, D, generator=g).half()
+    slots = torch.randperm(NB * P, generator=g)[:T].int()
+    base_k = torch.randn(NB, Hkv * D // 16, P, 16, generator=g).half()  # pre-existing cache contents
+    base_v = torch.randn(NB, Hkv * D // 16, P, 16, generator=g).half()
+    kc_ref, vc_ref = base_k.clone(), base_v.clone()
+    R.reshape_and_cache_ref(key, kc_ref, slots, value, vc_ref)
+    kc, vc = base_k.to(dev), base_v.to(dev)
+    ops.reshape_and_cache(key.to(dev), value.to(dev), kc, vc, slots.to(dev))
+    # bit-exact including -0.0 / NaN payloads: compare the raw 16-bit patterns
+    assert torch.equal(kc.cpu().view(torch.int16), kc_ref.view(torch.int16))
+    assert torch.equal(vc.cpu().view(torch.int16), vc_ref.view(torch.int16))
+
+
+def test_reshape_and_cache_skips_bad_slots_and_roundtrips(ops, dev):
+    g = _gen(1)
+    NB, P, Hkv, D = 6, 32, 4, 128
+    dense = torch.randn(NB, P, Hkv, D, generator=g).half()
+    slots = torch.randperm(NB * P, generator=g).int()
+    key = dense.reshape(NB * P, Hkv, D)[slots.long()]
+    kc = torch.zeros(NB, Hkv * D // 16, P, 16, dtype=H, device=dev)
+    ops.reshape_and_cache(key.to(dev), None, kc, None, slots.to(dev))
+    assert torch.equal(kc.cpu(), R.nz_pack(dense))  # filling every slot == packing the dense tensor
+    kc.zero_()
+    bad = torch.tensor([-1, NB * P, 2**31 - 1, -(2**31), 5], dtype=torch.int32)
+    ops.reshape_and_cache(key[:5].to(dev), key[:5].to(dev), kc, kc.clone(), bad.to(dev))
+    got = kc.cpu()
+    assert torch.equal(got[0, :, 5, :].reshape(-1), key[4].reshape(-1))
+    got[0, :, 5, :] = 0
+    assert torch.count_nonzero(got) == 0
+
+
+# ----------------------------------------------------------------------------- grouped_matmul
+def _gmm_case(rows, K, N, E, seed, counts=None, wstd=0.02):
+    g = _gen(seed)
+    x = torch.randn(rows, K, generator=g).half()
+    w = (wstd * torch.randn(E, N, K, generator=g)).half().transpose(1, 2)
+    if counts is None:
+        ids = torch.randint(0, E, (rows,), generator=g)
+        gl = R.make_group_list(ids, E)
+    else:
+        gl = torch.tensor(counts).cumsum(0).to(torch.int64)
+    return x, w, gl
+
+
+@pytest.mark.parametrize(
+    "rows,K,N,E,counts",
+    [
+        (1024, 256, 256, 8, None),
+        (300, 64, 64, 4, [0, 1, 170, 129]),        # empty group, single row, >1 tile, minimum K and N
+        (513, 128, 192, 3, [128, 256, 100]),        # exact tile, two tiles, rows past the last group
+        (96, 2048, 1536, 1, [96]),                  # E = 1: plain GEMM
+        (700, 768, 2048, 5, [0, 0, 700, 0, 0]),     # everything in one expert
+        (64, 512, 64, 130, None),                   # more experts than lanes in a wave
+    ],
+)
+def test_grouped_matmul(ops, dev, rows, K, N, E, counts):
+    x, w, gl = _gmm_case(rows, K, N, E, seed=0, counts=counts)
+    sentinel = 77.0
+    ref = R.grouped_matmul_ref(x, w, gl, out=torch.full((rows, N), sentinel).half())
+    y = ops.grouped_matmul(x.to(dev), w.to(dev), gl.to(dev))
+    assert y.shape == (rows, N) and y.dtype == H
+    end = int(gl[-1])
+    torch.testing.assert_close(y.cpu()[:end].float(), ref[:end].float(), **GMM_TOL)
+
+
+def test_grouped_matmul_reference_script_shape(ops, dev):
+    # benchmark/test_grouped_matmul.py:28-50: 16384 x 2048 -> 768, 128 experts, multinomial routing
+    g = _gen(0)
+    rows, K, N, E = 16384, 2048, 768, 128
+    x = torch.randn(rows, K, generator=g).half()
+    w = (0.02 * torch.randn(E, N, K, generator=g)).half().transpose(1, 2)
+    sample = torch.multinomial(torch.ones(E), num_samples=rows, replacement=True, generator=g)
+    gl = torch.bincount(sample, minlength=E).cumsum(0).to(torch.int64)
+    y = ops.grouped_matmul(x.to(dev), w.to(dev), gl.to(dev))
+    ref = R.grouped_matmul_ref(x, w, gl)
+    torch.testing.assert_close(y.cpu().float(), ref.float(), **GMM_TOL)
+
+
+def test_grouped_matmul_does_not_write_past_the_last_group(ops, dev):
+    x, w, gl = _gmm_case(256, 128, 128, 2, seed=3, counts=[50, 60])
+    import ascend910a_extras.ascend910a_extras_C as C
+    y = torch.full((256, 128), 5.0, dtype=H, device=dev)
+    xd, wd, gd = x.to(dev), w.to(dev), gl.to(dev)
+    code = C._lib.aops_grouped_matmul_f16(xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y.data_ptr(), 256, 128, 2, 128,
+                                          torch.cuda.current_stream().cuda_stream)
+    assert code == 0
+    assert torch.all(y[110:] == 5.0)
+    ref = R.grouped_matmul_ref(x, w, gl)
+    torch.testing.assert_close(y.cpu()[:110].float(), ref[:110].float(), **GMM_TOL)
+
+
+def test_dense_mlp_chain(ops, dev):
+    """benchmark/test_mlp.py:37-41 through grouped_matmul with one expert (reduced width)."""
+    g = _gen(0)
+    bs, hidden, inter = 256, 1024, 3584
+    x = torch.randn(bs, hidden, generator=g).half()
+    gu = (0.02 * torch.randn(2 * inter, hidden, generator=g)).half()
+    dn = (0.02 * torch.randn(hidden, inter, generator=g)).half()
+    gl = torch.tensor([bs], dtype=torch.int64).to(dev)
+    h = ops.grouped_matmul(x.to(dev), gu.to(dev)[None].transpose(1, 2), gl)
+    h = ops.swiglu(h)
+    y = ops.grouped_matmul(h, dn.to(dev)[None].transpose(1, 2), gl)
+    torch.testing.assert_close(y.cpu().float(), R.mlp_ref(x, gu, dn).float(), **GMM_TOL)
+
+
+# ----------------------------------------------------------------------------- paged attention
+def _paged_case(B, Hq, Hkv, D, P, lens, seed, max_pages=None, extra_pages=5, poison=False):
+    g = _gen(seed)
+    pages_per = [(l + P - 1) // P for l in lens]
+    max_pages = max_pages or max(max(pages_per), 1)
+    NB = sum(pages_per) + extra_pages
+    perm = torch.randperm(NB, generator=g)
+    bt = torch.full((B, max_pages), -1 if poison else 0, dtype=torch.int32)
+    c = 0
+    used = torch.zeros(NB, P, dtype=torch.bool)
+    for b, n in enumerate(pages_per):
+        bt[b, :n] = perm[c:c + n].int()
+        for j in range(lens[b]):
+            used[int(bt[b, j // P]), j % P] = True
+        c += n
+    kd = torch.randn(NB, P, Hkv, D, generator=g).half()
+    vd = torch.randn(NB, P, Hkv, D, generator=g).half()
+    if poison:
+        kd[~used] = float("nan")
+        vd[~used] = float("nan")
+    q = torch.randn(B, Hq, D, generator=g).half()
+    return q, R.nz_pack(kd), R.nz_pack(vd), bt, torch.tensor(lens, dtype=torch.int32)
+
+
+def _run_pa(ops, dev, case):
+    q, kc, vc, bt, cl = case
+    return ops.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), bt.to(dev), cl.to(dev)).cpu()
+
+
+@pytest.mark.parametrize(
+    "B,Hq,Hkv,P,lens",
+    [
+        (4, 32, 8, 128, [512, 4096, 1000, 37]),
+        (6, 32, 8, 128, [1, 2, 31, 32, 33, 129]),
+        (3, 8, 8, 32, [100, 1, 700]),          # no GQA, small pages
+        (2, 16, 8, 64, [64, 65]),               # group of 2
+        (2, 16, 2, 128, [300, 2049]),           # group of 8
+        (3, 32, 8, 128, [0, 128, 0]),           # empty sequences
+    ],
+)
+def test_paged_attention(ops, dev, B, Hq, Hkv, P, lens):
+    case = _paged_case(B, Hq, Hkv, 128, P, lens, seed=0)
+    o = _run_pa(ops, dev, case)
+    ref = R.paged_attention_ref(*case)
+    assert o.shape == (B, Hq, 128) and o.dtype == H
+    torch.testing.assert_close(o.float(), ref.float(), **TOL)
+    # the op's error is far below the bar: typical |o| ~ 0.05, so also check a tight absolute error
+    assert (o.float() - ref.float()).abs().max() < 2e-3
+
+
+def test_paged_attention_ignores_garbage_and_unused_table_entries(ops, dev):
+    lens = [5, 130, 257, 1]
+    clean = _paged_case(4, 32, 8, 128, 128, lens, seed=1, max_pages=6)
+    dirty = _paged_case(4, 32, 8, 128, 128, lens, seed=1, max_pages=6, poison=True)
+    o_clean = _run_pa(ops, dev, clean)
+    o_dirty = _run_pa(ops, dev, dirty)
+    assert not torch.isnan(o_dirty).any()
+    assert torch.equal(o_clean, o_dirty)
+
+
+def test_paged_attention_special_cases(ops, dev):
+    q, kc, vc, bt, cl = _paged_case(3, 32, 8, 128, 128, [1, 640, 200], seed=2)
+    o = _run_pa(ops, dev, (q, kc, vc, bt, cl))
+    # L = 1 -> o = V_0 exactly (softmax weight 1)
+    v0 = R.gather_kv_from_cache(vc, bt[0], 1, 8)[0]
+    for h in range(32):
+        assert torch.equal(o[0, h], v0[h // 4])
+    # identical queries inside a GQA group give identical outputs
+    q2 = q.clone(); q2[:, 1] = q2[:, 0]
+    o2 = _run_pa(ops, dev, (q2, kc, vc, bt, cl))
+    assert torch.equal(o2[:, 0], o2[:, 1])
+    # permuting physical pages together with the table changes nothing (bitwise)
+    NB = kc.shape[0]
+    perm = torch.randperm(NB, generator=_gen(5))
+    inv = torch.empty_like(perm); inv[perm] = torch.arange(NB)
+    o3 = _run_pa(ops, dev, (q, kc[perm], vc[perm], inv[bt.long()].int(), cl))
+    assert torch.equal(o3, o)
+    # large scores: keys aligned with the query must not overflow the softmax
+    q4 = (q * 6).half()
+    kd = R.nz_unpack(kc, 8); j = 77
+    kd[int(bt[1, 0]), j] = q4[1, ::4] * 1.0
+    o4 = _run_pa(ops, dev, (q4, R.nz_pack(kd), vc, bt, cl))
+    ref4 = R.paged_attention_ref(q4, R.nz_pack(kd), vc, bt, cl)
+    assert torch.isfinite(o4).all()
+    torch.testing.assert_close(o4.float(), ref4.float(), **TOL)
+
+
+def test_decode_step_pipeline(ops, dev):
+    """rope -> reshape_and_cache of the new token at position ctx-1 -> paged attention, in the
+    order of the reference's decoder layer (csrc/ffi/graph.cpp:255-358)."""
+    g = _gen(0)
+    B, Hq, Hkv, D, P = 8, 32, 8, 128, 128
+    lens = torch.randint(1, 1500, (B,), generator=g).tolist()
+    q, kc, vc, bt, cl = _paged_case(B, Hq, Hkv, D, P, lens, seed=4)
+    k_new = torch.randn(B, Hkv, D, generator=g).half()
+    v_new = torch.randn(B, Hkv, D, generator=g).half()
+    cos, sin = R.build_cos_sin_cache(4096, D, theta=1e6)
+    pos = (cl - 1).int()
+    slots = torch.tensor([int(bt[b, int(pos[b]) // P]) * P + int(pos[b]) % P for b in range(B)], dtype=torch.int32)
+    # oracle
+    rq, rk = R.rope_ref(q, k_new, pos, cos, sin)
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    R.reshape_and_cache_ref(rk, kc_ref, slots, v_new, vc_ref)
+    o_ref = R.paged_attention_ref(rq, kc_ref, vc_ref, bt, cl)
+    # device
+    kcd, vcd = kc.to(dev), vc.to(dev)
+    oq, ok = ops.rope(q.to(dev), k_new.to(dev), pos.to(dev), cos.to(dev), sin.to(dev))
+    ops.reshape_and_cache(ok, v_new.to(dev), kcd, vcd, slots.to(dev))
+    o = ops.paged_attention(oq, kcd, vcd, bt.to(dev), cl.to(dev))
+    assert torch.equal(vcd.cpu(), vc_ref)
+    torch.testing.assert_close(o.cpu().float(), o_ref.float(), **TOL)
+
+
+def test_ops_run_on_the_current_stream(ops, dev):
+    """The launchers enqueue on torch's current stream (reference: getCurrentNPUStream)."""
+    x = torch.randn(64, 256, device=dev, dtype=H)
+    s = torch.cuda.Stream(device=dev)
+    s.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(s):
+        y = ops.swiglu(x)
+    s.synchronize()
+    torch.testing.assert_close(y.cpu().float(), R.swiglu_ref(x.cpu()).float(), **TOL)
+
+
+def test_print_info(ops, dev, capsys):
+    ops.print_info()
+    out = capsys.readouterr().out
+    assert "compute units" in out and "gfx" in out

@@ -1,0 +1,285 @@
+"""Pins the CPU oracle (oracle/ops_ref.py) without a GPU: the reference's own
+known-answer case, closed forms, library routines and invariants, chosen so
+that a dropped term, a wrong sign/index or a transposed operand fails."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle.ops_ref as R
+
+
+# ----------------------------------------------------------------------------- add_rms_norm
+def test_add_rms_norm_matches_library_rms_norm():
+    torch.manual_seed(0)
+    x = torch.randn(16, 256).half()
+    r = torch.randn(16, 256).half()
+    w = (1 + 0.1 * torch.randn(256)).half()
+    y, res = R.add_rms_norm_ref(x, r, w, 1e-6)
+    t = (x + r)
+    lib = torch.nn.functional.rms_norm(t.float(), (256,), w.float(), 1e-6)
+    torch.testing.assert_close(y.float(), lib, rtol=2e-3, atol=2e-3)
+    assert torch.equal(res, t)  # residual_out is the fp16 sum, bit for bit
+    # the fp16 sum equals the correctly rounded fp32 sum
+    assert torch.equal(res, (x.float() + r.float()).half())
+
+
+def test_add_rms_norm_invariants():
+    torch.manual_seed(1)
+    x = torch.randn(8, 128).half()
+    r = torch.randn(8, 128).half()
+    ones = torch.ones(128).half()
+    y, _ = R.add_rms_norm_ref(x, r, ones, 0.0)
+    torch.testing.assert_close((y.float() ** 2).mean(-1), torch.ones(8), rtol=5e-3, atol=5e-3)
+    # scale invariance for eps = 0 (power-of-two scale is exact in fp16)
+    y2, _ = R.add_rms_norm_ref(x * 4, r * 4, ones, 0.0)
+    torch.testing.assert_close(y2.float(), y.float(), rtol=2e-3, atol=2e-3)
+    # a zero row gives zeros (eps keeps the division finite)
+    z = torch.zeros(1, 128).half()
+    yz, rz = R.add_rms_norm_ref(z, z, ones, 1e-6)
+    assert torch.count_nonzero(yz) == 0 and torch.count_nonzero(rz) == 0
+    # hand-computed: t = [3, 4, 0, 0...] over H=64 -> mean sq = 25/64, rms = 5/8
+    x1 = torch.zeros(1, 64).half(); x1[0, 0] = 1; x1[0, 1] = 3
+    r1 = torch.zeros(1, 64).half(); r1[0, 0] = 2; r1[0, 1] = 1
+    w1 = torch.full((64,), 2.0).half()
+    y1, t1 = R.add_rms_norm_ref(x1, r1, w1, 0.0)
+    assert t1[0, 0] == 3 and t1[0, 1] == 4
+    torch.testing.assert_close(y1[0, :2].float(), torch.tensor([3 / 0.625 * 2, 4 / 0.625 * 2]), rtol=1e-3, atol=1e-3)
+
+
+# ----------------------------------------------------------------------------- swiglu
+def test_swiglu_against_library_silu_and_special_cases():
+    torch.manual_seed(2)
+    x = torch.randn(32, 256).half()
+    y = R.swiglu_ref(x)
+    lib = torch.nn.functional.silu(x[:, :128].float()) * x[:, 128:].float()
+    torch.testing.assert_close(y.float(), lib, rtol=1e-3, atol=1e-3)
+    # second half == 1 -> silu of the first half (a swapped-halves bug would give x1*sigmoid(1)... )
+    x1 = x.clone(); x1[:, 128:] = 1
+    torch.testing.assert_close(R.swiglu_ref(x1).float(), torch.nn.functional.silu(x[:, :128].float()), rtol=1e-3, atol=1e-3)
+    # first half == 0 -> 0 regardless of the second half
+    x0 = x.clone(); x0[:, :128] = 0
+    assert torch.count_nonzero(R.swiglu_ref(x0)) == 0
+    # it is NOT the other convention (x1 * sigmoid(x2)) that the reference script also holds
+    other = x[:, :128].float() * torch.sigmoid(x[:, 128:].float())
+    assert (y.float() - other).abs().max() > 0.1
+    # numeric spot value: silu(2)*3 = 2/(1+e^-2)*3
+    xs = torch.tensor([[2.0] * 32 + [3.0] * 32]).half()
+    assert abs(float(R.swiglu_ref(xs)[0, 0]) - 6 / (1 + math.exp(-2))) < 5e-3
+
+
+# ----------------------------------------------------------------------------- rope
+def test_cos_sin_cache_values():
+    cos, sin = R.build_cos_sin_cache(64, 128, theta=1e6)
+    assert cos.shape == (64, 64) and sin.shape == (64, 64) and cos.dtype == torch.float16
+    for pos, i in [(0, 0), (1, 0), (5, 3), (63, 63), (17, 32)]:
+        ang = pos * (1e6 ** (-2 * i / 128))
+        assert abs(float(cos[pos, i]) - math.cos(ang)) < 1e-3
+        assert abs(float(sin[pos, i]) - math.sin(ang)) < 1e-3
+
+
+def test_rope_closed_form_and_invariants():
+    torch.manual_seed(3)
+    B, Hq, Hkv, D = 5, 4, 2, 64
+    q = torch.randn(B, Hq, D).half(); k = torch.randn(B, Hkv, D).half()
+    cos, sin = R.build_cos_sin_cache(128, D, theta=1e4)
+    pos = torch.tensor([0, 1, 7, 100, 127], dtype=torch.int32)
+    oq, ok = R.rope_ref(q, k, pos, cos, sin)
+    # position 0 is the identity
+    assert torch.equal(oq[0], q[0]) and torch.equal(ok[0], k[0])
+    # complex multiplication (x_i + i x_{i+h}) * (cos + i sin)
+    h = D // 2
+    zc = torch.complex(q[..., :h].float(), q[..., h:].float())
+    rot = torch.complex(cos[pos.long()].float(), sin[pos.long()].float())[:, None, :]
+    z = zc * rot
+    want = torch.cat([z.real, z.imag], -1)
+    torch.testing.assert_close(oq.float(), want, rtol=2e-3, atol=2e-3)
+    # pairwise norms are preserved
+    n_in = k[..., :h].float() ** 2 + k[..., h:].float() ** 2
+    n_out = ok[..., :h].float() ** 2 + ok[..., h:].float() ** 2
+    torch.testing.assert_close(n_out, n_in, rtol=1e-2, atol=1e-2)
+    # rotating back with the negated sine table returns the input
+    bq, _ = R.rope_ref(oq, ok, pos, cos, -sin)
+    torch.testing.assert_close(bq.float(), q.float(), rtol=1e-2, atol=1e-2)
+    # the native-dtype evaluation (what the reference script does) agrees within fp16 tolerance
+    nq, nk = R.rope_ref(q, k, pos, cos, sin, compute_dtype=torch.float16)
+    torch.testing.assert_close(nq.float(), oq.float(), rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(nk.float(), ok.float(), rtol=1e-2, atol=1e-2)
+
+
+# ----------------------------------------------------------------------------- reshape_and_cache
+def test_reshape_and_cache_reference_known_answer():
+    """The reference's own CPU-reproducible case (benchmark/test_reshape_and_cache.py:29-42):
+    seed 42, 4 tokens, cache [583, 64, 128, 16], slots [6, 134, 212, 290]."""
+    torch.manual_seed(42)
+    slots = torch.tensor([6, 134, 212, 290], dtype=torch.int32)
+    key = torch.randn(4, 8, 128, dtype=torch.float16)
+    value = torch.randn(4, 8, 128, dtype=torch.float16)
+    kc = torch.zeros(583, 64, 128, 16, dtype=torch.float16)
+    vc = torch.zeros_like(kc)
+    R.reshape_and_cache_ref(key, kc, slots, value, vc)
+    # blocks [0,1,1,2], offsets [6,6,84,34]; element f of a token's row sits at [f // 16, off, f % 16]
+    for t, (blk, off) in enumerate([(0, 6), (1, 6), (1, 84), (2, 34)]):
+        assert torch.equal(kc[blk, :, off, :].reshape(-1), key[t].reshape(-1))
+        assert torch.equal(vc[blk, :, off, :].reshape(-1), value[t].reshape(-1))
+        for f in (0, 15, 16, 129, 1023):
+            assert kc[blk, f // 16, off, f % 16] == key[t].reshape(-1)[f]
+    assert int(torch.count_nonzero(kc)) == int(torch.count_nonzero(key))
+    # the literal-loop transcription agrees bit for bit
+    kc2 = torch.zeros_like(kc); vc2 = torch.zeros_like(kc)
+    R.reshape_and_cache_loop(key, kc2, slots, value, vc2)
+    assert torch.equal(kc, kc2) and torch.equal(vc, vc2)
+    # key-only call leaves the value cache untouched (benchmark/test_reshape_and_cache.py:73-83)
+    kc3 = torch.zeros_like(kc); vc3 = torch.zeros_like(kc)
+    R.reshape_and_cache_ref(key, kc3, slots)
+    assert torch.equal(kc3, kc) and torch.count_nonzero(vc3) == 0
+
+
+def test_reshape_and_cache_pack_roundtrip_and_skips():
+    torch.manual_seed(4)
+    NB, P, H, D = 3, 32, 2, 64
+    dense = torch.randn(NB, P, H, D).half()
+    cache = R.nz_pack(dense)
+    assert cache.shape == (NB, H * D // 16, P, 16)
+    assert torch.equal(R.nz_unpack(cache, H), dense)
+    # writing every slot through reshape_and_cache reproduces nz_pack
+    slots = torch.randperm(NB * P).int()
+    key = dense.reshape(NB * P, H, D)[slots.long()]
+    kc = torch.zeros_like(cache)
+    R.reshape_and_cache_ref(key, kc, slots)
+    assert torch.equal(kc, cache)
+    # negative and too-large slots are skipped
+    kc = torch.zeros_like(cache)
+    bad = torch.tensor([-1, NB * P, 5], dtype=torch.int32)
+    R.reshape_and_cache_ref(key[:3], kc, bad)
+    assert int(torch.count_nonzero(kc[0, :, 5, :])) > 0
+    kc[0, :, 5, :] = 0
+    assert torch.count_nonzero(kc) == 0
+
+
+# ----------------------------------------------------------------------------- grouped_matmul
+def test_grouped_matmul_reduces_to_library_gemm_and_handles_groups():
+    torch.manual_seed(5)
+    R_, K, N, E = 40, 64, 128, 4
+    x = torch.randn(R_, K).half()
+    w = (0.05 * torch.randn(E, N, K)).half().transpose(1, 2)  # logical [E, K, N], K-major storage
+    # E = 1: plain GEMM
+    y1 = R.grouped_matmul_ref(x, w[:1], torch.tensor([R_]))
+    torch.testing.assert_close(y1.float(), x.float() @ w[0].float(), rtol=2e-3, atol=2e-3)
+    # groups: [0,7) e0, empty e1, [7,8) e2 (one row), [8,33) e3; rows 33.. untouched
+    gl = torch.tensor([7, 7, 8, 33], dtype=torch.int64)
+    out = torch.full((R_, N), 7.0).half()
+    y = R.grouped_matmul_ref(x, w, gl, out=out)
+    for e, (s, t) in enumerate([(0, 7), (7, 7), (7, 8), (8, 33)]):
+        if t > s:
+            want = np.asarray(x[s:t].float()) @ np.asarray(w[e].float())  # numpy as second opinion
+            np.testing.assert_allclose(np.asarray(y[s:t].float()), want, rtol=2e-3, atol=2e-3)
+    assert torch.all(y[33:] == 7.0)
+    # a transposed-operand mistake would not even have the right shape: w[e] is [K, N]
+    assert w[0].shape == (K, N) and w.stride(1) == 1 and w.stride(2) == K
+
+
+def test_make_group_list_and_mlp():
+    ids = torch.tensor([3, 0, 0, 2, 3, 3])
+    assert R.make_group_list(ids, 5).tolist() == [2, 2, 3, 6, 6]
+    torch.manual_seed(6)
+    x = torch.randn(4, 64).half()
+    gu = (0.1 * torch.randn(256, 64)).half()
+    dn = (0.1 * torch.randn(64, 128)).half()
+    y = R.mlp_ref(x, gu, dn)
+    h = x.float() @ gu.float().T
+    h = (torch.nn.functional.silu(h[:, :128]) * h[:, 128:])
+    torch.testing.assert_close(y.float(), h @ dn.float().T, rtol=2e-2, atol=2e-2)
+
+
+# ----------------------------------------------------------------------------- paged attention
+def _make_paged(B, Hq, Hkv, D, P, lens, seed, nb_extra=3):
+    g = torch.Generator().manual_seed(seed)
+    pages_per = [(l + P - 1) // P for l in lens]
+    max_pages = max(max(pages_per), 1)
+    NB = sum(pages_per) + nb_extra
+    perm = torch.randperm(NB, generator=g)
+    bt = torch.zeros(B, max_pages, dtype=torch.int32)
+    c = 0
+    for b, n in enumerate(pages_per):
+        bt[b, :n] = perm[c:c + n].int(); c += n
+    kd = torch.randn(NB, P, Hkv, D, generator=g).half()
+    vd = torch.randn(NB, P, Hkv, D, generator=g).half()
+    q = torch.randn(B, Hq, D, generator=g).half()
+    return q, kd, vd, bt, torch.tensor(lens, dtype=torch.int32)
+
+
+def _dense_attention(q, kd, vd, bt, lens):
+    """Independent computation from the dense [NB, P, Hkv, D] tensors with per-head loops."""
+    B, Hq, D = q.shape
+    P, Hkv = kd.shape[1], kd.shape[2]
+    out = torch.zeros(B, Hq, D)
+    for b in range(B):
+        L = int(lens[b])
+        if L == 0:
+            continue
+        K = torch.cat([kd[int(p)] for p in bt[b, :(L + P - 1) // P]])[:L].float()
+        V = torch.cat([vd[int(p)] for p in bt[b, :(L + P - 1) // P]])[:L].float()
+        for h in range(Hq):
+            g = h // (Hq // Hkv)
+            s = (K[:, g] @ q[b, h].float()) / math.sqrt(D)
+            p = torch.exp(s - s.max()); p = p / p.sum()
+            out[b, h] = p @ V[:, g]
+    return out
+
+
+def test_paged_attention_against_dense_layout_computation():
+    q, kd, vd, bt, lens = _make_paged(4, 8, 2, 32, 16, [1, 16, 37, 0], seed=7)
+    o = R.paged_attention_ref(q, R.nz_pack(kd), R.nz_pack(vd), bt, lens)
+    want = _dense_attention(q, kd, vd, bt, lens)
+    torch.testing.assert_close(o.float(), want, rtol=2e-3, atol=2e-3)
+    assert torch.count_nonzero(o[3]) == 0  # empty sequence
+
+
+def test_paged_attention_special_cases():
+    q, kd, vd, bt, lens = _make_paged(3, 4, 2, 32, 16, [1, 40, 23], seed=8)
+    kc, vc = R.nz_pack(kd), R.nz_pack(vd)
+    o = R.paged_attention_ref(q, kc, vc, bt, lens)
+    # L = 1: the output is V_0 of the sequence's kv head
+    v0 = vd[int(bt[0, 0]), 0]  # [Hkv, D]
+    for h in range(4):
+        assert torch.equal(o[0, h], v0[h // 2])
+    # all keys equal -> uniform weights -> mean of V
+    kd2 = kd.clone(); kd2[:] = kd[0, 0][None, None]
+    o2 = R.paged_attention_ref(q, R.nz_pack(kd2), vc, bt, lens)
+    L = 40
+    V = torch.cat([vd[int(p)] for p in bt[1, :3]])[:L].float()
+    torch.testing.assert_close(o2[1, 0].float(), V[:, 0].mean(0), rtol=2e-3, atol=2e-3)
+    # GQA: heads 0,1 share kv head 0 -> identical outputs for identical queries
+    q3 = q.clone(); q3[:, 1] = q3[:, 0]
+    o3 = R.paged_attention_ref(q3, kc, vc, bt, lens)
+    assert torch.equal(o3[:, 0], o3[:, 1])
+    assert not torch.equal(o3[:, 0], o3[:, 2])
+    # permuting the physical pages together with the block table changes nothing
+    NB = kd.shape[0]
+    perm = torch.randperm(NB, generator=torch.Generator().manual_seed(9))
+    inv = torch.empty_like(perm); inv[perm] = torch.arange(NB)
+    o4 = R.paged_attention_ref(q, R.nz_pack(kd[perm]), R.nz_pack(vd[perm]), inv[bt.long()].int(), lens)
+    assert torch.equal(o4, o)
+    # garbage past the end of a sequence (and in unused pages) is ignored
+    kd5, vd5 = kd.clone(), vd.clone()
+    used = set()
+    for b in range(3):
+        for j in range(int(lens[b])):
+            used.add((int(bt[b, j // 16]), j % 16))
+    for p in range(NB):
+        for off in range(16):
+            if (p, off) not in used:
+                kd5[p, off] = float("nan"); vd5[p, off] = float("nan")
+    o5 = R.paged_attention_ref(q, R.nz_pack(kd5), R.nz_pack(vd5), bt, lens)
+    assert torch.equal(o5, o)
+
+
+def test_paged_attention_one_dominant_key():
+    q, kd, vd, bt, lens = _make_paged(1, 2, 1, 32, 16, [30], seed=10)
+    j = 21
+    page, off = int(bt[0, j // 16]), j % 16
+    kd[page, off, 0] = q[0, 0] * 8  # score ~ 8*|q|^2/sqrt(D) dominates
+    o = R.paged_attention_ref(q, R.nz_pack(kd), R.nz_pack(vd), bt, lens)
+    torch.testing.assert_close(o[0, 0].float(), vd[page, off, 0].float(), rtol=1e-2, atol=1e-2)
