@@ -1,0 +1,603 @@
+#!/usr/bin/env python3
+"""Benchmark of the ascend910a_extras operator set on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|pa|gmm|...] [--no-cpu]
+
+A "step" is one paged_attention decode call over the batch of BASELINE.json configs[4]
+(64 sequences, 32 query / 8 kv heads, head_dim 128, contexts ~U[512, 4096], block 128): the
+largest HBM-bound workload of the operator set and the one the printed `value` is quoted on.
+Every other configuration is measured as well and reported under `per_op` of the same JSON line
+(add_rms_norm, reshape_and_cache, swiglu and the two dense GEMMs of the MLP, the MoE grouped GEMMs,
+rope, plus clearly labelled scaled shapes of the small operators).
+
+Timing:
+  * `ms_per_step` / `value`: wall clock around exactly K eager steps through the Python API,
+    bracketed by torch.cuda.synchronize() on both sides, inputs resident in HBM.
+  * `roofline` and `per_op[*].gpu_us`: HIP events (on the stream the kernels are launched on)
+    around replays of a HIP graph that holds one launch per rotating buffer set, so that
+    back-to-back kernels are timed rather than the host's launch rate; the buffer sets are
+    sized so that the footprint between two uses of the same buffer exceeds the 256 MB Infinity
+    Cache.  Algorithmic bytes = every input read once, every output written once.
+  * `cpu_baseline` / `per_op[*].cpu_ms`: the CPU oracle (plain torch, fp32 math) on the same
+    inputs on this machine's host cores, median of a few runs.  The oracle is the checker and
+    the timed baseline only; nothing measured on the GPU goes through it.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import math
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "ascend-ops_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
+CACHE_BYTES = 320 << 20      # Infinity Cache (256 MB) + L2, what a rotation has to exceed
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+# --------------------------------------------------------------------------------------- timing
+def _events_ms(fn, reps):
+    import torch
+
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1)
+
+
+def time_graph(calls, min_launches=200, trials=5):
+    """Per-launch GPU time (microseconds) of `calls` (one closure per buffer set), measured with
+    HIP events around replays of a graph that holds every closure once."""
+    import torch
+
+    for c in calls:
+        c()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for c in calls:
+            c()
+    reps = max(1, -(-min_launches // len(calls)))
+    graph.replay()
+    per = []
+    for _ in range(trials):
+        per.append(_events_ms(graph.replay, reps) * 1e3 / (reps * len(calls)))
+    del graph
+    return statistics.median(per), min(per)
+
+
+def time_eager(calls, warmup, iters):
+    import torch
+
+    n = len(calls)
+    for i in range(warmup):
+        calls[i % n]()
+    it = iter(range(10**9))
+    ms = _events_ms(lambda: calls[next(it) % n](), iters)
+    return ms * 1e3 / iters
+
+
+def time_cpu(fn, runs=3):
+    fn()
+    ts = []
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return statistics.median(ts) * 1e3
+
+
+def n_sets_for(bytes_per_set, lo=2, hi=128):
+    return int(max(lo, min(hi, math.ceil(CACHE_BYTES / max(bytes_per_set, 1)) + 1)))
+
+
+# --------------------------------------------------------------------------------------- C ABI
+class Lib:
+    """Direct C-ABI launches on preallocated buffers (kernel timing without allocator effects)."""
+
+    def __init__(self):
+        import torch
+        import ascend910a_extras.ascend910a_extras_C as C
+
+        self.lib = C._lib
+        self.torch = torch
+
+    def stream(self):
+        return self.torch.cuda.current_stream().cuda_stream
+
+    def check(self, code):
+        if code != 0:
+            raise RuntimeError(self.lib.aops_strerror(code).decode())
+
+
+def entry(op, config, shape, bound, alg_bytes, alg_flops, gpu_us, gpu_us_min, eager_us, cpu_ms, cores, note=None):
+    e = {
+        "op": op, "config": config, "shape": shape, "bound": bound,
+        "algorithmic_bytes": alg_bytes, "algorithmic_flops": alg_flops,
+        "gpu_us": round(gpu_us, 3), "gpu_us_min": round(gpu_us_min, 3),
+        "api_eager_us": None if eager_us is None else round(eager_us, 3),
+    }
+    gbps = alg_bytes / (gpu_us * 1e-6) / 1e9
+    e["GBps"] = round(gbps, 1)
+    e["hbm_frac"] = round(gbps / HBM_PEAK_GBPS, 4)
+    if alg_flops:
+        tf = alg_flops / (gpu_us * 1e-6) / 1e12
+        e["TFLOPs"] = round(tf, 1)
+        e["mfma_frac"] = round(tf / MFMA_F16_PEAK_TFLOPS, 4)
+    if cpu_ms is not None:
+        e["cpu_ms"] = round(cpu_ms, 3)
+        e["cpu_cores"] = cores
+        e["gpu_over_cpu"] = round(cpu_ms * 1e3 / gpu_us, 1)
+    if note:
+        e["note"] = note
+    return e
+
+
+# --------------------------------------------------------------------------------------- workloads
+def bench_add_rms_norm(L, ops, R, dev, cpu, T, config, note=None):
+    import torch
+
+    Hd, eps = 4096, 1e-6
+    torch.manual_seed(0)
+    x = torch.randn(T, Hd).half()
+    r = torch.randn(T, Hd).half()
+    w = (1 + 0.1 * torch.randn(Hd)).half()
+    alg = 4 * T * Hd * 2 + Hd * 2
+    n = n_sets_for(alg)
+    xs = [x.to(dev).clone() for _ in range(n)]
+    rs = [r.to(dev).clone() for _ in range(n)]
+    ys = [torch.empty_like(xs[0]) for _ in range(n)]
+    os_ = [torch.empty_like(xs[0]) for _ in range(n)]
+    wd = w.to(dev)
+
+    def mk(i):
+        return lambda: L.check(L.lib.aops_add_rms_norm_f16(xs[i].data_ptr(), rs[i].data_ptr(), wd.data_ptr(), eps,
+                                                          ys[i].data_ptr(), os_[i].data_ptr(), T, Hd, L.stream()))
+
+    calls = [mk(i) for i in range(n)]
+    med, mn = time_graph(calls)
+    eager = time_eager([(lambda i=i: ops.add_rms_norm(xs[i], rs[i], wd, eps)) for i in range(n)], 10, 100)
+    y_ref, res_ref = R.add_rms_norm_ref(x, r, w, eps)
+    torch.testing.assert_close(ys[-1].cpu().float(), y_ref.float(), rtol=1e-2, atol=1e-2)
+    assert torch.equal(os_[-1].cpu(), res_ref)
+    cpu_ms = time_cpu(lambda: R.add_rms_norm_ref(x, r, w, eps)) if cpu else None
+    return entry("add_rms_norm", config, f"x,residual [{T},{Hd}] f16", "hbm", alg, 0, med, mn, eager, cpu_ms,
+                 torch.get_num_threads(), note)
+
+
+def bench_swiglu(L, ops, R, dev, cpu, T, d, config, note=None):
+    import torch
+
+    torch.manual_seed(0)
+    x = torch.randn(T, 2 * d).half()
+    alg = T * d * 2 * 3
+    n = n_sets_for(alg)
+    xs = [x.to(dev).clone() for _ in range(n)]
+    ys = [torch.empty(T, d, dtype=torch.float16, device=dev) for _ in range(n)]
+
+    def mk(i):
+        return lambda: L.check(L.lib.aops_swiglu_f16(xs[i].data_ptr(), ys[i].data_ptr(), T, d, L.stream()))
+
+    med, mn = time_graph([mk(i) for i in range(n)])
+    eager = time_eager([(lambda i=i: ops.swiglu(xs[i])) for i in range(n)], 10, 100)
+    torch.testing.assert_close(ys[-1].cpu().float(), R.swiglu_ref(x).float(), rtol=1e-2, atol=1e-2)
+    cpu_ms = time_cpu(lambda: R.swiglu_ref(x)) if cpu else None
+    return entry("swiglu", config, f"x [{T},{2 * d}] f16", "hbm", alg, 0, med, mn, eager, cpu_ms,
+                 torch.get_num_threads(), note)
+
+
+def bench_rope(L, ops, R, dev, cpu, B, config, note=None):
+    import torch
+
+    Hq, Hkv, D, max_pos = 32, 8, 128, 4096
+    torch.manual_seed(0)
+    q = torch.randn(B, Hq, D).half()
+    k = torch.randn(B, Hkv, D).half()
+    pos = torch.randint(511, 4096, (B,), dtype=torch.int32)
+    cos, sin = R.build_cos_sin_cache(max_pos, D, theta=1e6)
+    alg = 2 * B * (Hq + Hkv) * D * 2 + B * 4 + 2 * B * (D // 2) * 2
+    n = n_sets_for(alg)
+    qs = [q.to(dev).clone() for _ in range(n)]
+    ks = [k.to(dev).clone() for _ in range(n)]
+    oq = [torch.empty_like(qs[0]) for _ in range(n)]
+    ok = [torch.empty_like(ks[0]) for _ in range(n)]
+    pd, cd, sd = pos.to(dev), cos.to(dev), sin.to(dev)
+
+    def mk(i):
+        return lambda: L.check(L.lib.aops_rope_neox_f16(qs[i].data_ptr(), ks[i].data_ptr(), pd.data_ptr(), cd.data_ptr(),
+                                                       sd.data_ptr(), oq[i].data_ptr(), ok[i].data_ptr(), B, Hq, Hkv, D,
+                                                       L.stream()))
+
+    med, mn = time_graph([mk(i) for i in range(n)])
+    eager = time_eager([(lambda i=i: ops.rope(qs[i], ks[i], pd, cd, sd)) for i in range(n)], 10, 100)
+    rq, rk = R.rope_ref(q, k, pos, cos, sin)
+    torch.testing.assert_close(oq[-1].cpu().float(), rq.float(), rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(ok[-1].cpu().float(), rk.float(), rtol=1e-2, atol=1e-2)
+    cpu_ms = time_cpu(lambda: R.rope_ref(q, k, pos, cos, sin)) if cpu else None
+    return entry("rope", config, f"q [{B},{Hq},{D}], k [{B},{Hkv},{D}] f16", "hbm", alg, 0, med, mn, eager, cpu_ms,
+                 torch.get_num_threads(), note)
+
+
+def bench_reshape_and_cache(L, ops, R, dev, cpu, T, config, note=None):
+    import torch
+
+    Hkv, D, NB, P = 8, 128, 1024, 128
+    torch.manual_seed(0)
+    key = torch.randn(T, Hkv, D).half()
+    value = torch.randn(T, Hkv, D).half()
+    slots = torch.randperm(NB * P)[:T].int()
+    alg = 4 * T * Hkv * D * 2 + T * 4
+    n = n_sets_for(alg, lo=2, hi=48)
+    n_cache = 2  # 2 x (2 x 256 MiB): a cache pair is reused only after 1 GiB of other lines
+    ks = [key.to(dev).clone() for _ in range(n)]
+    vs = [value.to(dev).clone() for _ in range(n)]
+    kcs = [torch.zeros(NB, Hkv * D // 16, P, 16, dtype=torch.float16, device=dev) for _ in range(n_cache)]
+    vcs = [torch.zeros(NB, Hkv * D // 16, P, 16, dtype=torch.float16, device=dev) for _ in range(n_cache)]
+    sd = slots.to(dev)
+
+    def mk(i):
+        c = i % n_cache
+        return lambda: L.check(L.lib.aops_reshape_and_cache_f16(ks[i].data_ptr(), vs[i].data_ptr(), kcs[c].data_ptr(),
+                                                               vcs[c].data_ptr(), sd.data_ptr(), T, Hkv * D, NB, P,
+                                                               L.stream()))
+
+    med, mn = time_graph([mk(i) for i in range(n)])
+    eager = time_eager([(lambda i=i: ops.reshape_and_cache(ks[i], vs[i], kcs[i % n_cache], vcs[i % n_cache], sd))
+                        for i in range(n)], 10, 100)
+    kc_ref = torch.zeros(NB, Hkv * D // 16, P, 16, dtype=torch.float16)
+    vc_ref = torch.zeros_like(kc_ref)
+    cpu_ms = None
+    if cpu:
+        cpu_ms = time_cpu(lambda: R.reshape_and_cache_ref(key, kc_ref, slots, value, vc_ref), runs=2 if T > 4096 else 3)
+    else:
+        R.reshape_and_cache_ref(key, kc_ref, slots, value, vc_ref)
+    assert torch.equal(kcs[0].cpu(), kc_ref) and torch.equal(vcs[0].cpu(), vc_ref), "reshape_and_cache not bit-exact"
+    return entry("reshape_and_cache", config, f"key,value [{T},{Hkv},{D}] -> caches [{NB},{Hkv * D // 16},{P},16] f16",
+                 "hbm", alg, 0, med, mn, eager, cpu_ms, torch.get_num_threads(), note)
+
+
+def _gmm_entry(L, ops, R, dev, cpu, op, config, x, w_storage, gl, note=None, check_rows=4096):
+    """x [rows,K] cpu f16, w_storage [E,N,K] cpu f16, gl int64 cumulative."""
+    import torch
+
+    rows, K = x.shape
+    E, N, _ = w_storage.shape
+    end = int(gl[-1])
+    flops = 2 * end * K * N
+    alg = rows * K * 2 + E * N * K * 2 + end * N * 2 + E * 8
+    xd, wd, gd = x.to(dev), w_storage.to(dev), gl.to(dev)
+    n = n_sets_for(alg, lo=1, hi=8)
+    xs = [xd] + [xd.clone() for _ in range(n - 1)]
+    ws = [wd] + [wd.clone() for _ in range(n - 1)]
+    ys = [torch.empty(rows, N, dtype=torch.float16, device=dev) for _ in range(n)]
+
+    def mk(i):
+        return lambda: L.check(L.lib.aops_grouped_matmul_f16(xs[i].data_ptr(), ws[i].data_ptr(), gd.data_ptr(),
+                                                            ys[i].data_ptr(), rows, K, E, N, L.stream()))
+
+    med, mn = time_graph([mk(i) for i in range(n)], min_launches=40)
+    eager = time_eager([(lambda i=i: ops.grouped_matmul(xs[i], ws[i].transpose(1, 2), gd)) for i in range(n)], 3, 20)
+    w_logical = w_storage.transpose(1, 2)
+    cpu_ms = None
+    if cpu:
+        t0 = time.perf_counter()
+        ref = R.grouped_matmul_ref(x, w_logical, gl)
+        cpu_ms = (time.perf_counter() - t0) * 1e3
+        torch.testing.assert_close(ys[-1].cpu()[:end].float(), ref[:end].float(), rtol=2e-2, atol=2e-2)
+    else:
+        # check a slice of rows only (first experts) to keep the run short
+        sub_end = min(end, check_rows)
+        e_hi = int((gl < sub_end).sum()) + 1
+        gsub = torch.clamp(gl[:e_hi], max=sub_end)
+        ref = R.grouped_matmul_ref(x[:sub_end], w_logical[:e_hi], gsub)
+        torch.testing.assert_close(ys[-1].cpu()[:sub_end].float(), ref.float(), rtol=2e-2, atol=2e-2)
+    e = entry(op, config, f"x [{rows},{K}] @ w [{E},{K},{N}] f16", "mfma", alg, flops, med, mn, eager, cpu_ms,
+              torch.get_num_threads(), note)
+    hbm_floor_us = alg / (HBM_PEAK_GBPS * 1e9) * 1e6
+    mfma_floor_us = flops / (MFMA_F16_PEAK_TFLOPS * 1e12) * 1e6
+    e["hbm_floor_us"] = round(hbm_floor_us, 2)
+    e["mfma_floor_us"] = round(mfma_floor_us, 2)
+    e["frac_of_roofline_ceiling"] = round(max(hbm_floor_us, mfma_floor_us) / med, 4)
+    return e, ys[-1]
+
+
+def bench_moe(L, ops, R, dev, cpu):
+    import torch
+
+    E, hidden, inter, tokens, topk = 128, 2048, 768, 4096, 8
+    torch.manual_seed(0)
+    rows = tokens * topk
+    ids = torch.randint(0, E, (rows,))
+    gl = R.make_group_list(ids, E)
+    x = torch.randn(rows, hidden).half()
+    w1 = torch.empty(E, 2 * inter, hidden, dtype=torch.float16)
+    w2 = torch.empty(E, hidden, inter, dtype=torch.float16)
+    for e in range(E):  # chunked generation keeps the fp32 temporaries small
+        w1[e] = (0.02 * torch.randn(2 * inter, hidden)).half()
+        w2[e] = (0.02 * torch.randn(hidden, inter)).half()
+    out = []
+    e1, h_dev = _gmm_entry(L, ops, R, dev, cpu, "grouped_matmul", "4: MoE gate_up", x, w1, gl)
+    out.append(e1)
+    del w1
+    h = ops.swiglu(h_dev)
+    # swiglu at the MoE shape
+    T, d = rows, inter
+    alg = T * d * 2 * 3
+    n = n_sets_for(alg)
+    hs = [h_dev.clone() for _ in range(n)]
+    ys = [torch.empty(T, d, dtype=torch.float16, device=dev) for _ in range(n)]
+    med, mn = time_graph([(lambda i=i: L.check(L.lib.aops_swiglu_f16(hs[i].data_ptr(), ys[i].data_ptr(), T, d, L.stream())))
+                          for i in range(n)])
+    h_cpu = h_dev.cpu()
+    cpu_ms = time_cpu(lambda: R.swiglu_ref(h_cpu)) if cpu else None
+    torch.testing.assert_close(ys[-1].cpu().float(), R.swiglu_ref(h_cpu).float(), rtol=1e-2, atol=1e-2)
+    out.append(entry("swiglu", "4: MoE activation", f"x [{T},{2 * d}] f16", "hbm", alg, 0, med, mn, None, cpu_ms,
+                     torch.get_num_threads()))
+    del hs, ys
+    e2, _ = _gmm_entry(L, ops, R, dev, cpu, "grouped_matmul", "4: MoE down", h.cpu(), w2, gl)
+    out.append(e2)
+    tot_flops = e1["algorithmic_flops"] + e2["algorithmic_flops"]
+    tot_us = e1["gpu_us"] + e2["gpu_us"]
+    out.append({
+        "op": "grouped_matmul", "config": "4: MoE gate_up + down (sum of the two GEMMs)",
+        "algorithmic_flops": tot_flops, "gpu_us": round(tot_us, 3),
+        "TFLOPs": round(tot_flops / tot_us / 1e6, 1),
+        "mfma_frac": round(tot_flops / tot_us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
+    })
+    return out
+
+
+def bench_mlp(L, ops, R, dev, cpu):
+    import torch
+
+    bs, hidden, inter = 256, 4096, 14336
+    torch.manual_seed(0)
+    x = torch.randn(bs, hidden).half()
+    gu = torch.empty(2 * inter, hidden, dtype=torch.float16)
+    for i in range(0, 2 * inter, 2048):
+        gu[i:i + 2048] = (0.02 * torch.randn(2048, hidden)).half()
+    dn = (0.02 * torch.randn(hidden, inter)).half()
+    gl = torch.tensor([bs], dtype=torch.int64)
+    out = []
+    e1, h_dev = _gmm_entry(L, ops, R, dev, cpu, "grouped_matmul (E=1)", "3: MLP gate_up GEMM", x, gu[None], gl,
+                           note="dense GEMM run as one expert; weight-stream bound, reported not scored")
+    out.append(e1)
+    out.append(bench_swiglu(L, ops, R, dev, cpu, bs, inter, "3: MLP swiglu"))
+    h = ops.swiglu(h_dev)
+    e2, y_dev = _gmm_entry(L, ops, R, dev, cpu, "grouped_matmul (E=1)", "3: MLP down GEMM", h.cpu(), dn[None], gl,
+                           note="dense GEMM run as one expert; weight-stream bound, reported not scored")
+    out.append(e2)
+    if cpu:
+        torch.testing.assert_close(y_dev.cpu().float(), R.mlp_ref(x, gu, dn).float(), rtol=2e-2, atol=2e-2)
+    return out
+
+
+class PagedAttentionWorkload:
+    """BASELINE.json configs[4]: decode attention with neox rope and the cache write of the new token."""
+
+    def __init__(self, R, dev, n_sets=2):
+        import torch
+
+        self.B, self.Hq, self.Hkv, self.D, self.P, self.NB = 64, 32, 8, 128, 128, 2304
+        B, Hq, Hkv, D, P, NB = self.B, self.Hq, self.Hkv, self.D, self.P, self.NB
+        torch.manual_seed(0)
+        self.ctx = torch.randint(512, 4097, (B,), dtype=torch.int32)
+        pages_per = ((self.ctx + P - 1) // P).tolist()
+        self.max_pages = 32
+        perm = torch.randperm(NB)
+        self.bt = torch.zeros(B, self.max_pages, dtype=torch.int32)
+        c = 0
+        for b, npg in enumerate(pages_per):
+            self.bt[b, :npg] = perm[c:c + npg].int()
+            c += npg
+        self.q = torch.randn(B, Hq, D).half()
+        self.k = torch.randn(B, Hkv, D).half()
+        self.v = torch.randn(B, Hkv, D).half()
+        self.kc = torch.empty(NB, Hkv * D // 16, P, 16, dtype=torch.float16)
+        self.vc = torch.empty_like(self.kc)
+        for i in range(0, NB, 64):  # chunked: keeps fp32 temporaries small
+            self.kc[i:i + 64] = torch.randn(min(64, NB - i), Hkv * D // 16, P, 16).half()
+            self.vc[i:i + 64] = torch.randn(min(64, NB - i), Hkv * D // 16, P, 16).half()
+        self.cos, self.sin = R.build_cos_sin_cache(4096, D, theta=1e6)
+        self.pos = (self.ctx - 1).int()
+        self.slots = torch.tensor([int(self.bt[b, int(self.pos[b]) // P]) * P + int(self.pos[b]) % P for b in range(B)],
+                                  dtype=torch.int32)
+        sum_ctx = int(self.ctx.sum())
+        self.sum_ctx = sum_ctx
+        self.alg_bytes = sum_ctx * Hkv * D * 2 * 2 + 2 * B * Hq * D * 2 + self.bt.numel() * 4 + B * 4
+        self.dev = dev
+        self.d = {}
+        for name in ("q", "k", "v", "cos", "sin", "pos", "slots", "bt", "ctx"):
+            self.d[name] = getattr(self, name).to(dev)
+        kcd, vcd = self.kc.to(dev), self.vc.to(dev)
+        self.kcs = [kcd] + [kcd.clone() for _ in range(n_sets - 1)]
+        self.vcs = [vcd] + [vcd.clone() for _ in range(n_sets - 1)]
+        self.n_sets = n_sets
+
+    def step(self, ops, i=0):
+        d = self.d
+        return ops.paged_attention(d["q"], self.kcs[i % self.n_sets], self.vcs[i % self.n_sets], d["bt"], d["ctx"])
+
+    def pipeline(self, ops, i=0):
+        d = self.d
+        oq, ok = ops.rope(d["q"], d["k"], d["pos"], d["cos"], d["sin"])
+        ops.reshape_and_cache(ok, d["v"], self.kcs[i % self.n_sets], self.vcs[i % self.n_sets], d["slots"])
+        return ops.paged_attention(oq, self.kcs[i % self.n_sets], self.vcs[i % self.n_sets], d["bt"], d["ctx"])
+
+
+def bench_paged_attention(L, ops, R, dev, cpu, wl):
+    import torch
+
+    B, Hq, Hkv, D, P = wl.B, wl.Hq, wl.Hkv, wl.D, wl.P
+    ws_bytes = L.lib.aops_paged_attention_workspace(B, Hq, Hkv, D, P, wl.max_pages)
+    wss = [torch.empty(ws_bytes, dtype=torch.uint8, device=dev) for _ in range(wl.n_sets)]
+    outs = [torch.empty(B, Hq, D, dtype=torch.float16, device=dev) for _ in range(wl.n_sets)]
+    d = wl.d
+
+    def mk(i):
+        return lambda: L.check(L.lib.aops_paged_attention_f16(
+            d["q"].data_ptr(), wl.kcs[i].data_ptr(), wl.vcs[i].data_ptr(), d["bt"].data_ptr(), d["ctx"].data_ptr(),
+            outs[i].data_ptr(), wss[i].data_ptr(), ws_bytes, B, Hq, Hkv, D, P, wl.max_pages, wl.NB, L.stream()))
+
+    med, mn = time_graph([mk(i) for i in range(wl.n_sets)], min_launches=40)
+    eager = time_eager([(lambda i=i: wl.step(ops, i)) for i in range(wl.n_sets)], 5, 40)
+    cpu_ms = None
+    ref = None
+    if cpu:
+        t0 = time.perf_counter()
+        ref = R.paged_attention_ref(wl.q, wl.kc, wl.vc, wl.bt, wl.ctx)
+        cpu_ms = (time.perf_counter() - t0) * 1e3
+        torch.testing.assert_close(outs[0].cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+    e = entry("paged_attention", "5: decode attention", f"q [{B},{Hq},{D}], caches [{wl.NB},{Hkv * D // 16},{P},16], "
+              f"sum(context)={wl.sum_ctx}", "hbm", wl.alg_bytes, 4 * wl.sum_ctx * Hq * D, med, mn, eager, cpu_ms,
+              torch.get_num_threads(), note="two kernels per call: split-KV partial + merge")
+    e.pop("TFLOPs", None)
+    e.pop("mfma_frac", None)
+    # whole decode step: rope -> cache write -> attention (graph of the three C-ABI calls via the API)
+    pipe = time_eager([(lambda i=i: wl.pipeline(ops, i)) for i in range(wl.n_sets)], 5, 40)
+    e["pipeline_rope_cache_attention_api_eager_us"] = round(pipe, 2)
+    return e
+
+
+# --------------------------------------------------------------------------------------- main
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--ops", default="all", help="comma list of: pa,norm,cache,mlp,moe,rope,scaled or all")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (every operator is independent per token, per "
+                 "(sequence, kv head) or per expert and shards without an internal exchange); use --gpus 1")
+
+    import torch
+
+    import ascend910a_extras.ops as ops      # the product; raises if libaops.so is missing
+    import oracle.ops_ref as R               # checker + timed CPU baseline only
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L = Lib()
+    cpu = not args.no_cpu
+    want = set(args.ops.split(","))
+    allops = "all" in want
+    cores = torch.get_num_threads()
+    log(f"[bench] device: {torch.cuda.get_device_name(0)}; host threads: {cores} (os.cpu_count()={os.cpu_count()})")
+    log(f"[bench] denominators: HBM {HBM_PEAK_GBPS} GB/s, fp16 MFMA {MFMA_F16_PEAK_TFLOPS} TFLOP/s")
+
+    per_op = []
+
+    def run(tag, fn):
+        if allops or tag in want:
+            t0 = time.perf_counter()
+            res = fn()
+            res = res if isinstance(res, list) else [res]
+            per_op.extend(res)
+            for r in res:
+                log(f"[bench] {json.dumps(r)}")
+            log(f"[bench] {tag} done in {time.perf_counter() - t0:.1f}s")
+            torch.cuda.empty_cache()
+
+    # ------------------------------------------------------------------ primary: paged attention
+    t0 = time.perf_counter()
+    wl = PagedAttentionWorkload(R, dev)
+    log(f"[bench] config 5 inputs ready in {time.perf_counter() - t0:.1f}s; sum(context)={wl.sum_ctx}")
+    for i in range(args.warmup):
+        wl.step(ops, i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        wl.step(ops, i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    pa = bench_paged_attention(L, ops, R, dev, cpu, wl)
+    log(f"[bench] {json.dumps(pa)}")
+    per_op.append(pa)
+    sum_ctx, alg_bytes = wl.sum_ctx, wl.alg_bytes
+    del wl
+    torch.cuda.empty_cache()
+
+    run("norm", lambda: bench_add_rms_norm(L, ops, R, dev, cpu, 128, "1: add_rms_norm"))
+    run("cache", lambda: bench_reshape_and_cache(L, ops, R, dev, cpu, 2048, "2: reshape_and_cache"))
+    run("rope", lambda: bench_rope(L, ops, R, dev, cpu, 64, "5: rope"))
+    run("mlp", lambda: bench_mlp(L, ops, R, dev, cpu))
+    run("moe", lambda: bench_moe(L, ops, R, dev, cpu))
+    run("scaled", lambda: [
+        bench_add_rms_norm(L, ops, R, dev, False, 16384, "1 scaled x128: add_rms_norm",
+                           "scaled shape: shows the kernel's asymptotic bandwidth, not a BASELINE config"),
+        bench_reshape_and_cache(L, ops, R, dev, False, 65536, "2 scaled x32: reshape_and_cache",
+                                "scaled shape: shows the kernel's asymptotic bandwidth, not a BASELINE config"),
+        bench_swiglu(L, ops, R, dev, False, 8192, 14336, "3 scaled x32: swiglu",
+                     "scaled shape: shows the kernel's asymptotic bandwidth, not a BASELINE config"),
+        bench_rope(L, ops, R, dev, False, 16384, "5 scaled x256: rope",
+                   "scaled shape: shows the kernel's asymptotic bandwidth, not a BASELINE config"),
+    ])
+
+    gbps_wall = alg_bytes / (ms_per_step * 1e-3) / 1e9
+    gbps_kernel = alg_bytes / (pa["gpu_us"] * 1e-6) / 1e9
+    line = {
+        "metric": "paged-attention decode HBM GB/s (algorithmic bytes / step); other operators under per_op",
+        "value": round(gbps_wall, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE configs[4]: paged-attention decode, batch 64, 32 q heads / 8 kv heads, head_dim 128, "
+                        "block 128, context ~U[512,4096], shuffled int32 block tables",
+            "sum_context_tokens": sum_ctx,
+            "algorithmic_bytes_per_step": alg_bytes,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(gbps_kernel, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "kernel": "pa_decode_partial + pa_decode_merge (one call)",
+            "us_per_call": pa["gpu_us"],
+        },
+        "cpu_baseline": None if not cpu else {
+            "value": round(alg_bytes / (pa["cpu_ms"] * 1e-3) / 1e9, 3),
+            "unit": "GB/s",
+            "cores": cores,
+            "kind": "port",
+            "sample": "the full configs[4] batch (64 sequences), one pass of the torch fp32 oracle",
+            "ms": pa["cpu_ms"],
+        },
+        "per_op": per_op,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
