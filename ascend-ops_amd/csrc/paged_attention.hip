@@ -8,27 +8,35 @@
 // read on the device only, so the grid is sized for the longest possible context and
 // workgroups past the end of their sequence exit at once.
 //
-// Data path of the main kernel (head_dim 128): for one kv head a page holds K as
-// [8 d-chunks][block_size tokens][16 halfs], i.e. 32-byte granules.  A lane owns the 8
-// consecutive d values  d = 8*(lane%16) ..+7  for good (its slice of q stays in registers,
-// its slice of the output accumulates in registers) and the four 16-lane rows of a wave take
-// four neighbouring tokens, so every 128-bit load instruction of a wave fetches eight whole
-// 128-byte lines and each cache byte is read exactly once.  q.K is finished with DPP adds
-// inside the 16-lane row (no LDS), every row keeps its own running softmax state, and rows,
-// waves and chunks are merged once at the end.  K and V of the next 32 tokens are in flight
-// while the current 32 are consumed.
+// Main kernel (head_dim 128), one step = 32 tokens of one kv head = 8 KiB of K + 8 KiB of V:
+//  * For one kv head a page holds K as [8 d-chunks][block_size tokens][16 halfs].  A lane
+//    (n = lane%16, kg = lane/16) loads, for token n of a 16-token group, the 16 bytes that hold
+//    d = 32s + 8kg ..+7 (s = 0..3).  That register IS the per-lane operand of
+//    v_mfma_f32_16x16x32_f16 (8 consecutive k per lane), so S^T[token][head] = K . Q^T runs on
+//    the matrix core straight from the loads, and every load instruction of a wave fetches
+//    two contiguous 512-byte runs.
+//  * The MFMA result leaves lane (head, kg) with the scores of tokens 4kg..4kg+3 of each group:
+//    after exp2 and packing that is already the per-lane operand P^T of the second product, so
+//    the softmax needs two cross-row exchanges per step (for the running maximum) and no LDS.
+//  * O^T[d][head] += V^T . P^T needs V with tokens along k.  V is loaded exactly like K and
+//    transposed on the matrix core: V_tile . Sel with a 0/1 selector matrix returns
+//    [token][16 d] blocks whose result layout has 4 consecutive tokens per lane; converted
+//    back to fp16 (exact) they are the V^T operand.
+//  * The K registers are refilled for the next step as soon as the scores are out, the V
+//    registers as soon as P.V is done; three workgroups per CU cover each other's waits.
 //
 // Semantics: signature, cache indexing, GQA mapping and the fixed 1/sqrt(D) scale follow
 // reference csrc/ffi/ops.cpp:408-482, csrc/opdev/op_host/paged_attention_ex.cpp:18-36 and
 // csrc/opdev/op_kernel/paged_attention_ex.cpp:90-99 (whose compute body is unfinished).
+#include <stdlib.h>
+
 #include "aops_common.h"
 
 namespace aops {
 
-constexpr int kPaD = 128;         // head_dim of the fast path
-constexpr int kPaWaves = 4;       // waves per workgroup
-constexpr int kPaLoads = 8;       // 128-bit loads per lane per step (each covers 4 tokens/wave)
-constexpr int kPaStep = 4 * kPaLoads;  // tokens per wave per step
+constexpr int kPaD = 128;     // head_dim of the fast path
+constexpr int kPaWaves = 4;   // waves per workgroup
+constexpr int kPaStep = 32;   // tokens per wave per step (two 16-token MFMA groups)
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -45,6 +53,12 @@ static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_si
   while (chunk > kPaWaves * kPaStep &&
          bs * num_kv_heads * ((max_len + chunk - 1) / chunk) < 1024)
     chunk /= 2;
+  static const int forced = [] {
+    const char* e = getenv("AOPS_PA_CHUNK");  // tuning aid; must be a multiple of 128
+    const int v = e ? atoi(e) : 0;
+    return (v >= kPaWaves * kPaStep && v % (kPaWaves * kPaStep) == 0) ? v : 0;
+  }();
+  if (forced) chunk = forced;
   PaChunking c;
   c.chunk_tokens = chunk;
   c.max_splits = (int)((max_len + chunk - 1) / chunk);
@@ -52,68 +66,91 @@ static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_si
   return c;
 }
 
-struct F16x8Pairs {
-  f16x2 p[4];
+// Per-lane slice of a 32-token tile: [token group][s] holds X[token 16t + n][d = 32s + 8kg ..+7].
+typedef f16x8 PaRegs[2][4];
+
+__device__ __forceinline__ void pa_issue_loads(const f16* __restrict__ base, uint32_t lane_off,
+                                               uint32_t s_stride, PaRegs& r) {
+#pragma unroll
+  for (int g = 0; g < 2; ++g)
+#pragma unroll
+    for (int s = 0; s < 4; ++s) r[g][s] = ld128_stream(base + lane_off + s * s_stride + g * 256);
+}
+
+struct PaState {
+  f32x4 o[8];  // O^T blocks: lane (head n, kg), o[db][i] <-> d = 16 db + 4 kg + i
+  float m;     // running maximum of head n (identical in the four lanes of a head)
+  float l;     // this lane's share of the running sum
 };
 
-template <int G, bool MASKED>
-__device__ __forceinline__ void pa_step(const f16x8 (&kreg)[kPaLoads], f16x8 (&vreg)[kPaLoads],
-                                        const f16x2 (&q2)[G][4], float scale_log2,
-                                        int first_token, int context_len, float (&m)[G],
-                                        float (&l)[G], float (&acc)[G][8]) {
-  float s[kPaLoads][G];
+// S^T[token][head] = K . Q^T, scaled to log2 units; lane (head n, kg) gets tokens
+// 16*(e/4) + 4kg + e%4, e = 0..7, of the step.
+__device__ __forceinline__ void pa_scores(const PaRegs& k, const f16x8 (&qreg)[4],
+                                          float scale_log2, float (&sc)[8]) {
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  f32x4 sacc[2] = {zero4, zero4};
 #pragma unroll
-  for (int i = 0; i < kPaLoads; ++i) {
-    const F16x8Pairs kp = __builtin_bit_cast(F16x8Pairs, kreg[i]);
+  for (int g = 0; g < 2; ++g)
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
-      float a = 0.f;
+    for (int s = 0; s < 4; ++s)
+      sacc[g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(k[g][s], qreg[s], sacc[g], 0, 0, 0);
 #pragma unroll
-      for (int c = 0; c < 4; ++c) a = __builtin_amdgcn_fdot2(kp.p[c], q2[h][c], a, false);
-      s[i][h] = row16_sum(a) * scale_log2;
-    }
-    if (MASKED) {
-      const bool valid = first_token + 4 * i < context_len;
+  for (int g = 0; g < 2; ++g)
 #pragma unroll
-      for (int h = 0; h < G; ++h) s[i][h] = valid ? s[i][h] : -__builtin_inff();
-      // Cache contents past the end of the sequence are arbitrary (possibly NaN).
-      const f16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-      vreg[i] = valid ? vreg[i] : zero;
-    }
+    for (int i = 0; i < 4; ++i) sc[4 * g + i] = sacc[g][i] * scale_log2;
+}
+
+// Online softmax update; returns the P^T operand (lane (head n, kg), element e <-> token e).
+__device__ __forceinline__ f16x8 pa_softmax(float (&sc)[8], PaState& st) {
+  float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                   fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+  mx = fmaxf(mx, __shfl_xor(mx, 16));
+  mx = fmaxf(mx, __shfl_xor(mx, 32));
+  const float m_new = fmaxf(st.m, mx);
+  const float alpha = __builtin_amdgcn_exp2f(st.m - m_new);
+  st.m = m_new;
+  f16x8 pt;
+  float psum = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    pt[e] = (f16)__builtin_amdgcn_exp2f(sc[e] - m_new);
+    psum += (float)pt[e];
   }
+  st.l = st.l * alpha + psum;
+  if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {  // the maximum rarely moves after the start
 #pragma unroll
-  for (int h = 0; h < G; ++h) {
-    float mx = m[h];
+    for (int db = 0; db < 8; ++db)
 #pragma unroll
-    for (int i = 0; i < kPaLoads; ++i) mx = fmaxf(mx, s[i][h]);
-    const float alpha = __builtin_amdgcn_exp2f(m[h] - mx);
-    m[h] = mx;
-    float psum = 0.f;
+      for (int i = 0; i < 4; ++i) st.o[db][i] *= alpha;
+  }
+  return pt;
+}
+
+// O^T += V^T . P^T with V transposed on the matrix core.
+__device__ __forceinline__ void pa_accumulate(const PaRegs& v, const f16x8 (&sel)[2], f16x8 pt,
+                                              PaState& st) {
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[h][j] *= alpha;
+  for (int s = 0; s < 4; ++s) {
 #pragma unroll
-    for (int i = 0; i < kPaLoads; ++i) {
-      const float p = __builtin_amdgcn_exp2f(s[i][h] - mx);
-      psum += p;
+    for (int u = 0; u < 2; ++u) {
+      // [token][d = 32s + 16u + n]: lane (n, kg) receives tokens 4kg..4kg+3 of each group
+      const f32x4 x0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(v[0][s], sel[u], zero4, 0, 0, 0);
+      const f32x4 x1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(v[1][s], sel[u], zero4, 0, 0, 0);
+      f16x8 vt;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc[h][j] += p * (float)vreg[i][j];
+      for (int i = 0; i < 4; ++i) {
+        vt[i] = (f16)x0[i];
+        vt[4 + i] = (f16)x1[i];
+      }
+      st.o[2 * s + u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt, pt, st.o[2 * s + u], 0, 0, 0);
     }
-    l[h] = l[h] * alpha + psum;
   }
 }
 
-__device__ __forceinline__ void pa_issue_loads(const f16* __restrict__ kbase,
-                                               const f16* __restrict__ vbase, uint32_t lane_off,
-                                               f16x8 (&kreg)[kPaLoads], f16x8 (&vreg)[kPaLoads]) {
-#pragma unroll
-  for (int i = 0; i < kPaLoads; ++i) kreg[i] = ld128_stream(kbase + lane_off + i * 64);
-#pragma unroll
-  for (int i = 0; i < kPaLoads; ++i) vreg[i] = ld128_stream(vbase + lane_off + i * 64);
-}
-
-// grid = (max_splits, Hkv, bs), block = 256.
+// grid = (max_splits, Hkv, bs), block = 256.  G = query heads per kv head (<= 16).
 template <int G>
-__global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
+__global__ __launch_bounds__(kPaWaves* kWave, 3) void pa_decode_partial(
     const f16* __restrict__ q, const f16* __restrict__ key_cache,
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ context_lens, float* __restrict__ part_o,
@@ -130,33 +167,36 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int lane = threadIdx.x & (kWave - 1);
-  const int row = lane >> 4;     // token row inside a load instruction
-  const int piece = lane & 15;   // 16-byte piece of the head: d = 8*piece ..+7
+  const int n = lane & 15;
+  const int kg = lane >> 4;
   const int num_heads = num_kv_heads * G;
 
-  // This lane's slice of the G query heads that share kv head g.
-  f16x2 q2[G][4];
+  // Q^T operand: lane (head n, kg) holds q[head n][32s + 8kg ..+7]; heads >= G are zero rows.
+  f16x8 qreg[4];
+  {
+    const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const f16* qp = q + ((int64_t)b * num_heads + g * G + (n < G ? n : 0)) * kPaD + 8 * kg;
 #pragma unroll
-  for (int h = 0; h < G; ++h) {
-    const F16x8Pairs qp = __builtin_bit_cast(
-        F16x8Pairs, ld128(q + ((int64_t)b * num_heads + g * G + h) * kPaD + piece * 8));
-#pragma unroll
-    for (int c = 0; c < 4; ++c) q2[h][c] = qp.p[c];
+    for (int s = 0; s < 4; ++s) qreg[s] = n < G ? ld128(qp + 32 * s) : zero8;
   }
-
-  float m[G], l[G], acc[G][8];
+  // Selector operands of the transposing product: sel[u][k][n] = (k == n + 16u), k = 8kg + e.
+  f16x8 sel[2];
 #pragma unroll
-  for (int h = 0; h < G; ++h) {
-    m[h] = kNegBig;
-    l[h] = 0.f;
+  for (int u = 0; u < 2; ++u)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[h][j] = 0.f;
-  }
+    for (int e = 0; e < 8; ++e) sel[u][e] = (8 * kg + e == n + 16 * u) ? (f16)1.0f : (f16)0.0f;
 
-  // Element offsets inside one page for this lane: d-chunk (piece/2) rows are block_size*16
-  // halfs apart, the two halves of a granule 8 halfs, neighbouring tokens 16 halfs.
-  const uint32_t lane_off = (uint32_t)(piece >> 1) * (uint32_t)block_size * 16u +
-                            (uint32_t)(piece & 1) * 8u + (uint32_t)row * 16u;
+  PaState st;
+#pragma unroll
+  for (int db = 0; db < 8; ++db) st.o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  st.m = kNegBig;
+  st.l = 0.f;
+
+  // Element offsets inside one page for this lane: d-chunk rows are block_size*16 halfs apart
+  // (this lane starts in row kg/2), the two halves of a granule 8 halfs, tokens 16 halfs.
+  const uint32_t lane_off = (uint32_t)(kg >> 1) * (uint32_t)block_size * 16u +
+                            (uint32_t)(kg & 1) * 8u + (uint32_t)n * 16u;
+  const uint32_t s_stride = 2u * (uint32_t)block_size * 16u;  // 32 d further = two d-chunk rows
   const int64_t page_elems = (int64_t)num_kv_heads * kPaD * block_size;
   const int64_t head_off = (int64_t)g * kPaD * block_size;
   const int32_t* table = block_tables + (int64_t)b * max_blocks_per_seq;
@@ -168,65 +208,59 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
     return page * page_elems + head_off + (int64_t)(tok - blk * block_size) * 16;
   };
 
-  f16x8 kcur[kPaLoads], vcur[kPaLoads], knext[kPaLoads], vnext[kPaLoads];
+  PaRegs kreg, vreg;
   int step = wave;
   if (step < nsteps) {
     const int64_t off = page_offset(step);
-    pa_issue_loads(key_cache + off, value_cache + off, lane_off, kcur, vcur);
+    pa_issue_loads(key_cache + off, lane_off, s_stride, kreg);
+    pa_issue_loads(value_cache + off, lane_off, s_stride, vreg);
   }
   while (step < nsteps) {
     const int next = step + kPaWaves;
-    if (next < nsteps) {
-      const int64_t off = page_offset(next);
-      pa_issue_loads(key_cache + off, value_cache + off, lane_off, knext, vnext);
-    }
-    const int first_token = chunk_start + step * kPaStep + row;
-    if (chunk_start + (step + 1) * kPaStep <= context_len) {
-      pa_step<G, false>(kcur, vcur, q2, scale_log2, first_token, context_len, m, l, acc);
-    } else {
-      pa_step<G, true>(kcur, vcur, q2, scale_log2, first_token, context_len, m, l, acc);
-    }
+    const bool has_next = next < nsteps;
+    const int64_t next_off = has_next ? page_offset(next) : 0;
+    const int step_token0 = chunk_start + step * kPaStep;
+    float sc[8];
+    pa_scores(kreg, qreg, scale_log2, sc);
+    // K registers are free again: the next step's K is in flight during softmax and P.V.
+    if (has_next) pa_issue_loads(key_cache + next_off, lane_off, s_stride, kreg);
+    if (step_token0 + kPaStep > context_len) {  // wave uniform: last, partial step of the sequence
+      // Cache contents past the end of the sequence are arbitrary (possibly NaN): drop their
+      // scores and zero their V rows before they reach the matrix core.
+      const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int i = 0; i < kPaLoads; ++i) {
-      kcur[i] = knext[i];
-      vcur[i] = vnext[i];
+      for (int g = 0; g < 2; ++g) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (step_token0 + 16 * g + 4 * kg + i >= context_len) sc[4 * g + i] = -__builtin_inff();
+        if (step_token0 + 16 * g + n >= context_len) {
+#pragma unroll
+          for (int s = 0; s < 4; ++s) vreg[g][s] = zero8;
+        }
+      }
     }
+    const f16x8 pt = pa_softmax(sc, st);
+    pa_accumulate(vreg, sel, pt, st);
+    if (has_next) pa_issue_loads(value_cache + next_off, lane_off, s_stride, vreg);
     step = next;
   }
 
-  // Merge the four token rows of the wave (every lane ends up with the merged state).
-#pragma unroll
-  for (int h = 0; h < G; ++h) {
-    float mx = fmaxf(m[h], __shfl_xor(m[h], 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float w = __builtin_amdgcn_exp2f(m[h] - mx);
-    float lw = l[h] * w;
-    lw += __shfl_xor(lw, 16);
-    lw += __shfl_xor(lw, 32);
-    m[h] = mx;
-    l[h] = lw;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      float a = acc[h][j] * w;
-      a += __shfl_xor(a, 16);
-      a += __shfl_xor(a, 32);
-      acc[h][j] = a;
-    }
-  }
+  // The four lanes of a head hold disjoint shares of the sum.
+  float l_head = st.l;
+  l_head += __shfl_xor(l_head, 16);
+  l_head += __shfl_xor(l_head, 32);
 
   // Merge the waves of the workgroup through LDS and emit one partial per query head.
   __shared__ float sm_acc[kPaWaves][G][kPaD];
   __shared__ float sm_m[kPaWaves][G];
   __shared__ float sm_l[kPaWaves][G];
-  if (row == 0) {
+  if (n < G) {
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) sm_acc[wave][h][piece * 8 + j] = acc[h][j];
-      if (piece == 0) {
-        sm_m[wave][h] = m[h];
-        sm_l[wave][h] = l[h];
-      }
+    for (int db = 0; db < 8; ++db)
+      *reinterpret_cast<f32x4*>(&sm_acc[wave][n][16 * db + 4 * kg]) = st.o[db];
+    if (kg == 0) {
+      sm_m[wave][n] = st.m;
+      sm_l[wave][n] = l_head;
     }
   }
   __syncthreads();
