@@ -48,11 +48,16 @@ struct PaChunking {
 static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_size,
                               int64_t max_blocks_per_seq) {
   const int64_t max_len = block_size * max_blocks_per_seq;
-  int chunk = 512;
-  // Small problems: shorter chunks so that the grid still covers the chip.
-  while (chunk > kPaWaves * kPaStep &&
-         bs * num_kv_heads * ((max_len + chunk - 1) / chunk) < 1024)
-    chunk /= 2;
+  // As few chunks per sequence as still give every CU two workgroups: each chunk costs a
+  // partial result and a workgroup prologue, and long chunks keep the load stream steady.
+  constexpr int kUnit = kPaWaves * kPaStep;
+  constexpr int64_t kWantedWorkgroups = 512;
+  int64_t splits = (kWantedWorkgroups + bs * num_kv_heads - 1) / (bs * num_kv_heads > 0 ? bs * num_kv_heads : 1);
+  const int64_t max_units = (max_len + kUnit - 1) / kUnit;
+  if (splits > max_units) splits = max_units;
+  if (splits < 1) splits = 1;
+  int chunk = (int)(((max_units + splits - 1) / splits) * kUnit);
+  if (chunk < kUnit) chunk = kUnit;
   static const int forced = [] {
     const char* e = getenv("AOPS_PA_CHUNK");  // tuning aid; must be a multiple of 128
     const int v = e ? atoi(e) : 0;
@@ -149,19 +154,26 @@ __device__ __forceinline__ void pa_accumulate(const PaRegs& v, const f16x8 (&sel
 }
 
 // grid = (max_splits, Hkv, bs), block = 256.  G = query heads per kv head (<= 16).
-template <int G>
+// FINAL: the chunk is the whole sequence, so the normalised output is written directly.
+template <int G, bool FINAL>
 __global__ __launch_bounds__(kPaWaves* kWave, 3) void pa_decode_partial(
     const f16* __restrict__ q, const f16* __restrict__ key_cache,
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ context_lens, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int num_kv_heads, int block_size, int max_blocks_per_seq,
+    float* __restrict__ part_ml, f16* __restrict__ out, int num_kv_heads, int block_size, int max_blocks_per_seq,
     int chunk_tokens, int max_splits, float scale_log2) {
   const int split = blockIdx.x;
   const int g = blockIdx.y;
   const int b = blockIdx.z;
   const int context_len = context_lens[b];
   const int chunk_start = split * chunk_tokens;
-  if (chunk_start >= context_len) return;
+  if (chunk_start >= context_len) {
+    if (FINAL) {  // empty sequence: zeros
+      for (int e = threadIdx.x; e < G * kPaD; e += kPaWaves * kWave)
+        out[((int64_t)b * num_kv_heads * G + g * G) * kPaD + e] = (f16)0.f;
+    }
+    return;
+  }
   const int chunk_len = min(context_len - chunk_start, chunk_tokens);
   const int nsteps = (chunk_len + kPaStep - 1) / kPaStep;
 
@@ -277,11 +289,15 @@ __global__ __launch_bounds__(kPaWaves* kWave, 3) void pa_decode_partial(
       lsum += sm_l[w][h] * wt;
       a += sm_acc[w][h][d] * wt;
     }
-    const int64_t slot = ((int64_t)b * num_heads + g * G + h) * max_splits + split;
-    part_o[slot * kPaD + d] = a;
-    if (d == 0) {
-      part_ml[slot * 2 + 0] = mx;
-      part_ml[slot * 2 + 1] = lsum;
+    if (FINAL) {
+      out[((int64_t)b * num_heads + g * G + h) * kPaD + d] = (f16)(lsum > 0.f ? a / lsum : 0.f);
+    } else {
+      const int64_t slot = ((int64_t)b * num_heads + g * G + h) * max_splits + split;
+      part_o[slot * kPaD + d] = a;
+      if (d == 0) {
+        part_ml[slot * 2 + 0] = mx;
+        part_ml[slot * 2 + 1] = lsum;
+      }
     }
   }
 }
@@ -322,10 +338,15 @@ static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t*
                       PaChunking ch, hipStream_t s) {
   const float scale_log2 = kLog2e / __builtin_sqrtf((float)kPaD);
   dim3 grid((unsigned)ch.max_splits, (unsigned)num_kv_heads, (unsigned)bs);
-  pa_decode_partial<G><<<grid, kPaWaves * kWave, 0, s>>>(q, kc, vc, bt, cl, part_o, part_ml,
-                                                         num_kv_heads, block_size,
-                                                         max_blocks_per_seq, ch.chunk_tokens,
-                                                         ch.max_splits, scale_log2);
+  if (ch.max_splits == 1) {
+    pa_decode_partial<G, true><<<grid, kPaWaves * kWave, 0, s>>>(
+        q, kc, vc, bt, cl, part_o, part_ml, o, num_kv_heads, block_size, max_blocks_per_seq,
+        ch.chunk_tokens, ch.max_splits, scale_log2);
+    return;
+  }
+  pa_decode_partial<G, false><<<grid, kPaWaves * kWave, 0, s>>>(
+      q, kc, vc, bt, cl, part_o, part_ml, o, num_kv_heads, block_size, max_blocks_per_seq,
+      ch.chunk_tokens, ch.max_splits, scale_log2);
   dim3 mgrid((unsigned)num_heads, (unsigned)bs);
   pa_decode_merge<<<mgrid, kPaD, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
                                          ch.max_splits);

@@ -54,9 +54,14 @@ def test_api_surface_matches_reference_ops_py():
 def test_workspace_query_without_gpu():
     import ascend910a_extras.ascend910a_extras_C as C
 
-    # config 5 shape: 64 x 32 heads, 8 kv heads, D=128, P=128, 32 pages -> 8 chunks of 512
+    # config 5 shape: 64 x 32 heads, 8 kv heads, D=128, P=128, 32 pages; one (max, sum, 128 floats)
+    # record per (sequence, head, chunk), the number of chunks being the library's choice
     n = C._lib.aops_paged_attention_workspace(64, 32, 8, 128, 128, 32)
-    assert n == 64 * 32 * 8 * 130 * 4
+    per_chunk = 64 * 32 * 130 * 4
+    assert n >= per_chunk and n % per_chunk == 0 and n // per_chunk <= 32
+    # a single short sequence is split into more chunks than a large batch
+    n1 = C._lib.aops_paged_attention_workspace(1, 32, 8, 128, 128, 32)
+    assert n1 // (32 * 130 * 4) > n // per_chunk
     assert C._lib.aops_paged_attention_workspace(64, 32, 8, 96, 128, 32) == 0  # unsupported head_dim
     assert C._lib.aops_paged_attention_workspace(64, 32, 8, 128, 24, 32) == 0  # unsupported page size
 
