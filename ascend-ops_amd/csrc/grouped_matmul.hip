@@ -14,14 +14,15 @@
 // Semantics: reference csrc/opdev/op_kernel/grouped_mat_mul_ex.cpp:27-44 (start/end from the
 // cumulative int64 group_list, empty groups skipped), matmul_core.h:42-68 (NT product, fp32
 // accumulate, fp16 result), benchmark/test_grouped_matmul.py:6-23.
+#include <stdlib.h>
+
+#include <type_traits>
+
 #include "aops_common.h"
 
 namespace aops {
 
-constexpr int kBM = 128;
-constexpr int kBN = 128;
-constexpr int kBK = 64;
-constexpr int kGmmThreads = 256;
+constexpr int kBK = 64;   // k extent of one LDS stage
 constexpr int kXcds = 8;
 
 struct GmmWork {
@@ -33,6 +34,7 @@ struct GmmWork {
 };
 
 // Maps a work index to (expert, m-tile, n-tile).  Executed redundantly by every wave.
+template <int kBM>
 __device__ __forceinline__ GmmWork gmm_find_work(const int64_t* __restrict__ group_list,
                                                  int num_experts, int64_t rows, int n_tiles,
                                                  int wg, int num_wg) {
@@ -108,105 +110,261 @@ __device__ __forceinline__ GmmWork gmm_find_work(const int64_t* __restrict__ gro
   return w;
 }
 
-// LDS tile [rows][kBK] halfs; 16-byte chunk c of row r is stored at chunk (c ^ (r & 7)) so that
-// the 128-bit fragment reads of 8 consecutive rows hit all banks.
-__device__ __forceinline__ int lds_off(int r, int c) { return r * kBK + ((c ^ (r & 7)) << 3); }
+// LDS tile [rows][kBK] halfs, 128 bytes per row.  16-byte chunk c of row r is stored in row
+// r ^ ((r >> 3) & 1) at chunk position c ^ (r & 7): the 128-bit fragment reads of 8 or of 16
+// consecutive rows (same c) then touch every bank once, whichever width the LDS serves per
+// cycle, and so do the staging writes (8 consecutive chunks of a row per 8 lanes).
+__device__ __forceinline__ int lds_off(int r, int c) {
+  return (r ^ ((r >> 3) & 1)) * kBK + ((c ^ (r & 7)) << 3);
+}
 
-__global__ __launch_bounds__(kGmmThreads) void grouped_matmul_kernel(
+// Workgroup tile BM x BN = (64*MB) x (64*NB), four waves arranged 2 x 2.  Wave (wm, wn) owns
+// the 32-row blocks wm, wm+2, wm+4, ... (interleaved, so that a group that fills only part of
+// the tile still splits evenly between the two wave rows) and the 32*NB columns starting at
+// wn*32*NB; its MB x NB accumulators of v_mfma_f32_32x32x16_f16 stay in registers for the
+// whole k loop.  The products are formed as W.x^T (weight fragment as the first operand): a lane
+// then holds 4 consecutive output columns of one output row, which the epilogue packs to
+// 8 bytes, transposes through LDS and writes with 128-bit row-contiguous stores.
+//
+// Software pipeline per k tile (kBK = 64):
+//   global -> registers, D tiles ahead (the loads of tile kt+1+D are issued in iteration kt),
+//   registers -> LDS stage (kt+1)&1 during iteration kt, one barrier per k tile,
+//   LDS -> MFMA fragments one 16-wide k step ahead of the matrix cores.
+template <int MB, int NB, int D>
+__global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
     const f16* __restrict__ x, const f16* __restrict__ w, const int64_t* __restrict__ group_list,
     f16* __restrict__ y, int64_t rows, int k, int num_experts, int n) {
-  __shared__ __attribute__((aligned(16))) f16 sa[kBM * kBK];
-  __shared__ __attribute__((aligned(16))) f16 sb[kBN * kBK];
+  constexpr int BM = 64 * MB;
+  constexpr int BN = 64 * NB;
+  constexpr int kThreads = 4 * kWave;
+  constexpr int kAChunks = BM * (kBK / 8) / kThreads;  // 16-byte chunks per thread and tile
+  constexpr int kBChunks = BN * (kBK / 8) / kThreads;
+  constexpr int kRowsPerPass = kThreads / 8;           // tile rows covered by one chunk per thread
+  constexpr int kSteps = kBK / 16;
+  static_assert(D == 1 || D == 2, "prefetch distance");
+  static_assert(kRowsPerPass % 16 == 0, "swizzle must be invariant under the row stride");
 
-  const int n_tiles = (n + kBN - 1) / kBN;
-  const GmmWork work = gmm_find_work(group_list, num_experts, rows, n_tiles, blockIdx.x, gridDim.x);
+  extern __shared__ __attribute__((aligned(16))) f16 smem[];
+  f16* sa = smem;                 // [2][BM * kBK]
+  f16* sb = smem + 2 * BM * kBK;  // [2][BN * kBK]
+
+  const int n_tiles = (n + BN - 1) / BN;
+  const GmmWork work =
+      gmm_find_work<BM>(group_list, num_experts, rows, n_tiles, blockIdx.x, gridDim.x);
   if (!work.valid) return;
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
-  const int wave = tid / kWave;
-  const int wm = wave >> 1;  // 2 x 2 waves, 64 x 64 each
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave >> 1;
   const int wn = wave & 1;
+  const int tile_rows = min(work.row_end - work.row_begin, BM);
+  // 32-row blocks of this wave that hold at least one real row (wave uniform, 0..MB)
+  const int live_blocks = (tile_rows + 31) / 32;
+  const int live = (live_blocks - wm + 1) / 2;
 
-  // Global -> register staging: thread handles chunk (row = tid/8 + 32*i, kc = tid%8).
+  // Global -> register staging: thread handles chunk (row = tid/8 + kRowsPerPass*i, kc = tid%8).
+  // Sources are a uniform 64-bit tile base plus a 32-bit per-lane offset; LDS destinations are
+  // one per-lane offset plus compile-time strides.
   const int ld_row = tid >> 3;
   const int ld_kc = tid & 7;
-  const f16* a_src[4];
-  const f16* b_src[4];
+  const f16* a_base = x + (int64_t)work.row_begin * k;
+  const f16* b_base = w + ((int64_t)work.expert * n + (int64_t)work.n_tile * BN) * k;
+  uint32_t a_off[kAChunks], b_off[kBChunks];
+  const int n_left = n - work.n_tile * BN;  // rows of w available to this tile (>= 64)
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int ar = work.row_begin + ld_row + 32 * i;
-    if (ar > work.row_end - 1) ar = work.row_end - 1;  // rows past the group: duplicate, never stored
-    a_src[i] = x + (int64_t)ar * k + ld_kc * 8;
-    int br = work.n_tile * kBN + ld_row + 32 * i;
-    if (br > n - 1) br = n - 1;  // n is a multiple of 64, not necessarily of the tile width
-    b_src[i] = w + ((int64_t)work.expert * n + br) * k + ld_kc * 8;
+  for (int i = 0; i < kAChunks; ++i) {
+    int ar = ld_row + kRowsPerPass * i;
+    if (ar > tile_rows - 1) ar = tile_rows - 1;  // rows past the group: duplicates, never stored
+    a_off[i] = (uint32_t)ar * (uint32_t)k + ld_kc * 8;
   }
+#pragma unroll
+  for (int i = 0; i < kBChunks; ++i) {
+    int br = ld_row + kRowsPerPass * i;
+    if (br > n_left - 1) br = n_left - 1;  // n is a multiple of 64, not necessarily of BN
+    b_off[i] = (uint32_t)br * (uint32_t)k + ld_kc * 8;
+  }
+  const int st_dst = lds_off(ld_row, ld_kc);
 
-  f32x16 acc[2][2];
+  f32x16 acc[MB][NB];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MB; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NB; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  f16x8 ra[4], rb[4];
+  f16x8 ra[D][kAChunks], rb[D][kBChunks];  // D tiles in flight
+  const int ktiles = k / kBK;
+
+  auto load_tile = [&](int slot, int kt) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    ra[i] = ld128(a_src[i]);
-    rb[i] = ld128(b_src[i]);
-  }
+    for (int i = 0; i < kAChunks; ++i) ra[slot][i] = ld128(a_base + kt * kBK + a_off[i]);
+#pragma unroll
+    for (int i = 0; i < kBChunks; ++i) rb[slot][i] = ld128(b_base + kt * kBK + b_off[i]);
+  };
+  auto store_tile = [&](int slot, int stage) {
+    f16* da = sa + stage * BM * kBK;
+    f16* db = sb + stage * BN * kBK;
+#pragma unroll
+    for (int i = 0; i < kAChunks; ++i)
+      *reinterpret_cast<f16x8*>(&da[st_dst + i * kRowsPerPass * kBK]) = ra[slot][i];
+#pragma unroll
+    for (int i = 0; i < kBChunks; ++i)
+      *reinterpret_cast<f16x8*>(&db[st_dst + i * kRowsPerPass * kBK]) = rb[slot][i];
+  };
 
   const int fm = lane & 31;  // fragment row inside a 32-row block
   const int fq = lane >> 5;  // which half of a 16-wide k step
-  const int ktiles = k / kBK;
-  for (int kt = 0; kt < ktiles; ++kt) {
-    __syncthreads();
+  // Fragment reads: block offsets are compile-time strides on top of one per-lane offset per k
+  // step (the swizzle depends on fm and on the chunk only).
+  int frag_off[kSteps];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      *reinterpret_cast<f16x8*>(&sa[lds_off(ld_row + 32 * i, ld_kc)]) = ra[i];
-      *reinterpret_cast<f16x8*>(&sb[lds_off(ld_row + 32 * i, ld_kc)]) = rb[i];
-    }
-    __syncthreads();
-    if (kt + 1 < ktiles) {
+  for (int st = 0; st < kSteps; ++st) frag_off[st] = lds_off(fm, st * 2 + fq);
+  const f16* sa_w = sa + wm * 32 * kBK;
+  const f16* sb_w = sb + wn * 32 * NB * kBK;
+
+  // One pipeline step with LIVE live row blocks.  SLOT = register slot that holds tile kt+1,
+  // STAGE = LDS stage of tile kt.  The staging traffic (LDS writes of tile kt+1, global loads of
+  // tile kt+1+D) and the fragment reads of the next k step are issued in front of each group of
+  // MFMAs, so that they complete under the matrix cores' shadow.  Past the end of the k loop the
+  // same code runs on the last tile again (valid memory, results never consumed) instead of
+  // branching.
+  auto iteration = [&](int kt, auto slot_c, auto stage_c, auto live_c) {
+    constexpr int SLOT = decltype(slot_c)::value;
+    constexpr int STAGE = decltype(stage_c)::value;
+    constexpr int LIVE = decltype(live_c)::value;
+    const int kload = min(kt + 1 + D, ktiles - 1) * kBK;
+    constexpr int kAPer = (kAChunks + kSteps - 1) / kSteps;
+    constexpr int kBPer = (kBChunks + kSteps - 1) / kSteps;
+    const f16* ca = sa_w + STAGE * BM * kBK;
+    const f16* cb = sb_w + STAGE * BN * kBK;
+    f16* da = sa + (STAGE ^ 1) * BM * kBK;
+    f16* db = sb + (STAGE ^ 1) * BN * kBK;
+    f16x8 fa[2][LIVE > 0 ? LIVE : 1], fb[2][NB];
+    auto load_frags = [&](int buf, int st) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        ra[i] = ld128(a_src[i] + (kt + 1) * kBK);
-        rb[i] = ld128(b_src[i] + (kt + 1) * kBK);
+      for (int j = 0; j < NB; ++j)
+        fb[buf][j] = *reinterpret_cast<const f16x8*>(&cb[frag_off[st] + j * 32 * kBK]);
+#pragma unroll
+      for (int i = 0; i < LIVE; ++i)
+        fa[buf][i] = *reinterpret_cast<const f16x8*>(&ca[frag_off[st] + i * 64 * kBK]);
+    };
+    __syncthreads();  // stage STAGE is complete; stage STAGE^1 is no longer being read
+    load_frags(0, 0);
+#pragma unroll
+    for (int st = 0; st < kSteps; ++st) {
+      if (st + 1 < kSteps) load_frags((st + 1) & 1, st + 1);
+#pragma unroll
+      for (int i = st * kAPer; i < (st + 1) * kAPer && i < kAChunks; ++i) {
+        *reinterpret_cast<f16x8*>(&da[st_dst + i * kRowsPerPass * kBK]) = ra[SLOT][i];
+        ra[SLOT][i] = ld128(a_base + kload + a_off[i]);
       }
-    }
 #pragma unroll
-    for (int s = 0; s < kBK / 16; ++s) {
-      f16x8 fa[2], fb[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        fa[i] = *reinterpret_cast<const f16x8*>(&sa[lds_off(wm * 64 + i * 32 + fm, s * 2 + fq)]);
-        fb[i] = *reinterpret_cast<const f16x8*>(&sb[lds_off(wn * 64 + i * 32 + fm, s * 2 + fq)]);
+      for (int i = st * kBPer; i < (st + 1) * kBPer && i < kBChunks; ++i) {
+        *reinterpret_cast<f16x8*>(&db[st_dst + i * kRowsPerPass * kBK]) = rb[SLOT][i];
+        rb[SLOT][i] = ld128(b_base + kload + b_off[i]);
       }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < LIVE; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < NB; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[st & 1][j], fa[st & 1][i],
+                                                             acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
+  };
+
+  load_tile(0, 0);
+  store_tile(0, 0);
+#pragma unroll
+  for (int t = 1; t <= D; ++t) load_tile(t % D, min(t, ktiles - 1));
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using SlotEven = std::integral_constant<int, 1 % D>;  // slot of tile kt+1 for even kt
+  using SlotOdd = std::integral_constant<int, 2 % D>;   // ... for odd kt
+  // tile t travels in register slot t % D and is consumed from LDS stage t & 1
+  auto k_loop = [&](auto live_c) {
+    int kt = 0;
+    for (; kt + 1 < ktiles; kt += 2) {
+      iteration(kt, SlotEven{}, I0{}, live_c);
+      iteration(kt + 1, SlotOdd{}, I1{}, live_c);
+    }
+    if (kt < ktiles) iteration(kt, SlotEven{}, I0{}, live_c);
+  };
+  // One branch-free instantiation of the k loop per number of live row blocks.
+  if (live >= MB) {
+    k_loop(std::integral_constant<int, MB>{});
+  } else if (MB > 1 && live == MB - 1) {
+    k_loop(std::integral_constant<int, (MB > 1 ? MB - 1 : 0)>{});
+  } else if (MB > 2 && live == MB - 2) {
+    k_loop(std::integral_constant<int, (MB > 2 ? MB - 2 : 0)>{});
+  } else if (live >= 1) {  // short groups: rarely worth a dedicated copy, use the next larger one
+    if (MB > 3 && live <= MB - 3) k_loop(std::integral_constant<int, (MB > 3 ? MB - 3 : 0)>{});
+  } else {
+    k_loop(std::integral_constant<int, 0>{});
   }
 
-  // C fragment: lane holds column (lane%32) and rows 8*(r/4) + 4*(lane/32) + r%4, r = 0..15.
+  // Epilogue.  acc[i][j][r]: output row 32*(wm+2i) + lane%32, output columns
+  // wn*32*NB + 32j + 8*(r/4) + 4*(lane/32) + r%4.  The C tile goes to LDS as [BM][BN] halfs in
+  // 8-byte pieces, piece c of row m at position c ^ ((m & 15) << 1) (write conflicts at most
+  // 2-way, 16-byte reads stay contiguous), and leaves as 128-bit row-contiguous global stores.
+  __syncthreads();  // all waves are done with the operand stages
+  f16* sc = smem;
+  constexpr int kPiecesPerRow = BN / 4;
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < MB; ++i) {
+    const int m = 32 * (wm + 2 * i) + fm;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = work.row_begin + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * fq + (r & 3);
-      if (row < work.row_end) {
+    for (int j = 0; j < NB; ++j) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int col = work.n_tile * kBN + wn * 64 + j * 32 + fm;
-          if (col < n) y[(int64_t)row * n + col] = (f16)acc[i][j][r];
-        }
+      for (int g = 0; g < 4; ++g) {
+        f16x4 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (f16)acc[i][j][4 * g + e];
+        const int piece = (wn * 32 * NB + 32 * j + 8 * g + 4 * fq) >> 2;
+        *reinterpret_cast<f16x4*>(&sc[m * BN + ((piece ^ ((m & 15) << 1)) << 2)]) = v;
       }
     }
   }
+  __syncthreads();
+  constexpr int kChunksPerRow = BN / 8;              // 16-byte chunks per tile row
+  constexpr int kRowsPerStorePass = kThreads / kChunksPerRow;
+  const int c16 = tid % kChunksPerRow;
+  const int col = work.n_tile * BN + c16 * 8;
+  if (col < n) {
+    for (int m = tid / kChunksPerRow; m < tile_rows; m += kRowsPerStorePass) {
+      const f16x8 v = *reinterpret_cast<const f16x8*>(&sc[m * BN + ((c16 ^ (m & 15)) << 3)]);
+      st128(y + (int64_t)(work.row_begin + m) * n + col, v);
+    }
+  }
+}
+
+template <int MB, int NB, int D>
+static int gmm_launch(const f16* x, const f16* w, const int64_t* group_list, f16* y, int64_t rows,
+                      int k, int num_experts, int n, hipStream_t stream) {
+  constexpr int BM = 64 * MB;
+  constexpr int BN = 64 * NB;
+  constexpr int kStageBytes = 2 * (BM + BN) * kBK * (int)sizeof(f16);
+  constexpr int kTileBytes = BM * BN * (int)sizeof(f16);
+  constexpr int kLds = kStageBytes > kTileBytes ? kStageBytes : kTileBytes;
+  static_assert(kLds <= 160 * 1024, "LDS budget");
+  const int64_t n_tiles = (n + BN - 1) / BN;
+  const int64_t max_m_tiles = (rows + BM - 1) / BM + num_experts;
+  int64_t grid = max_m_tiles * n_tiles;
+  grid = (grid + kXcds - 1) / kXcds * kXcds;
+  if (grid > 0x7fffffff) return AOPS_ERR_INVALID_ARGUMENT;
+  auto kernel = grouped_matmul_kernel<MB, NB, D>;
+  static bool attr_set = false;  // benign race: the call is idempotent
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return record_launch_status(e);
+    attr_set = true;
+  }
+  kernel<<<(unsigned)grid, 4 * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts, n);
+  return record_launch_status(hipGetLastError());
 }
 
 }  // namespace aops
@@ -217,17 +375,30 @@ extern "C" int aops_grouped_matmul_f16(const void* x, const void* w, const int64
   using namespace aops;
   if (rows < 0 || k <= 0 || n <= 0 || num_experts < 0 || k % 64 != 0 || n % 64 != 0)
     return AOPS_ERR_INVALID_ARGUMENT;
-  if (rows > 0x7fffffff - kBM || k > 0x7fffffff || n > 0x7fffffff || num_experts > (1 << 20))
+  if (rows > 0x7fffffff - 4096 || k > 0x7fffffff || n > 0x7fffffff || num_experts > (1 << 20))
     return AOPS_ERR_INVALID_ARGUMENT;
   if (rows == 0 || num_experts == 0) return AOPS_OK;
   if (!x || !w || !group_list || !y) return AOPS_ERR_INVALID_ARGUMENT;
-  const int64_t n_tiles = (n + kBN - 1) / kBN;
-  const int64_t max_m_tiles = (rows + kBM - 1) / kBM + num_experts;
-  int64_t grid = max_m_tiles * n_tiles;
-  grid = (grid + kXcds - 1) / kXcds * kXcds;
-  if (grid > 0x7fffffff) return AOPS_ERR_INVALID_ARGUMENT;
-  grouped_matmul_kernel<<<(unsigned)grid, kGmmThreads, 0, static_cast<hipStream_t>(stream)>>>(
-      static_cast<const f16*>(x), static_cast<const f16*>(w), group_list, static_cast<f16*>(y),
-      rows, (int)k, (int)num_experts, (int)n);
-  return record_launch_status(hipGetLastError());
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const f16* xp = static_cast<const f16*>(x);
+  const f16* wp = static_cast<const f16*>(w);
+  f16* yp = static_cast<f16*>(y);
+  static const int variant = [] {
+    const char* e = getenv("AOPS_GMM_VARIANT");  // tuning aid
+    return e ? atoi(e) : 0;
+  }();
+  switch (variant) {
+    case 1:
+      return gmm_launch<2, 2, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
+    case 2:
+      return gmm_launch<4, 2, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
+    case 3:
+      return gmm_launch<5, 2, 1>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
+    case 4:
+      return gmm_launch<5, 2, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
+    case 5:
+      return gmm_launch<4, 4, 1>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
+    default:
+      return gmm_launch<5, 2, 1>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
+  }
 }
