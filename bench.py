@@ -480,10 +480,13 @@ def bench_paged_attention(L, ops, R, dev, cpu, wl):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--ops", default="all", help="comma list of: pa,norm,cache,mlp,moe,rope,scaled or all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--calib", action="store_true",
+                    help="also run a plain elementwise copy of 512 MiB (reads 512 MiB, writes 512 MiB): the known-size "
+                         "kernel against which FETCH_SIZE / WRITE_SIZE counters of a profiler run are scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (every operator is independent per token, per "
@@ -555,6 +558,23 @@ def main():
                    "scaled shape: shows the kernel's asymptotic bandwidth, not a BASELINE config"),
     ])
 
+    if args.calib:
+        src = torch.ones(256 << 20, dtype=torch.float16, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)  # one vectorized elementwise kernel: 512 MiB in, 512 MiB out
+        torch.cuda.synchronize()
+        log("[bench] calibration copy done: 3 launches, 536870912 B read + 536870912 B written each")
+        del src, dst
+
+    # HBM bytes per launch measured with rocprofv3 counters (recorded summary; None if absent)
+    traffic = None
+    tfile = os.path.join(ROOT, "profiles", "pa_decode_config5_hbm_traffic.txt")
+    if os.path.exists(tfile):
+        for ln in open(tfile):
+            if ln.strip().startswith("traffic_bytes_per_launch:"):
+                traffic = int(ln.split(":")[1])
+
     gbps_wall = alg_bytes / (ms_per_step * 1e-3) / 1e9
     gbps_kernel = alg_bytes / (pa["gpu_us"] * 1e-6) / 1e9
     line = {
@@ -582,8 +602,10 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4),
-            "traffic": None,
-            "kernel": "pa_decode_partial + pa_decode_merge (one call)",
+            "traffic": traffic,
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size; "
+                              "recorded in profiles/pa_decode_config5_hbm_traffic.txt" if traffic else None,
+            "kernel": "pa_decode_partial (split-KV main kernel; the merge kernel runs only when a sequence is split)",
             "us_per_call": pa["gpu_us"],
         },
         "cpu_baseline": None if not cpu else {
