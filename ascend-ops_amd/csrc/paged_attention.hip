@@ -2,7 +2,7 @@
 //
 //   o[b,h] = softmax_j( q[b,h] . K[j,g] / sqrt(D) ) . V[j,g],   g = h / (Hq/Hkv)
 //
-// Split-KV ("flash decoding"): a workgroup of 4 waves owns one (sequence, kv head, chunk of
+// Split-KV ("flash decoding"): a workgroup of 8 waves owns one (sequence, kv head, chunk of
 // the context); partial (max, sum, weighted V) triples go to a workspace and a second small
 // kernel merges the chunks of each (sequence, query head).  context_lens and block_tables are
 // read on the device only, so the grid is sized for the longest possible context and
@@ -35,7 +35,7 @@
 namespace aops {
 
 constexpr int kPaD = 128;     // head_dim of the fast path
-constexpr int kPaWaves = 4;   // waves per workgroup
+constexpr int kPaWaves = 8;   // waves per workgroup
 constexpr int kPaStep = 32;   // tokens per wave per step (two 16-token MFMA groups)
 constexpr float kNegBig = -1.0e30f;
 constexpr float kLog2e = 1.4426950408889634f;
@@ -156,7 +156,7 @@ __device__ __forceinline__ void pa_accumulate(const PaRegs& v, const f16x8 (&sel
 // grid = (max_splits, Hkv, bs), block = 256.  G = query heads per kv head (<= 16).
 // FINAL: the chunk is the whole sequence, so the normalised output is written directly.
 template <int G, bool FINAL>
-__global__ __launch_bounds__(kPaWaves* kWave, 3) void pa_decode_partial(
+__global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
     const f16* __restrict__ q, const f16* __restrict__ key_cache,
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ context_lens, float* __restrict__ part_o,
@@ -164,7 +164,22 @@ __global__ __launch_bounds__(kPaWaves* kWave, 3) void pa_decode_partial(
     int chunk_tokens, int max_splits, float scale_log2) {
   const int split = blockIdx.x;
   const int g = blockIdx.y;
-  const int b = blockIdx.z;
+  // Workgroups are handed out in index order, so they take the sequences longest first: with
+  // one resident workgroup per CU the short sequences then fill the gaps the long ones leave
+  // (longest-processing-time-first).  For batches of up to 64 sequences every wave finds the
+  // sequence of rank blockIdx.z by comparing the lengths held one per lane.
+  int b = blockIdx.z;
+  if (gridDim.z <= kWave) {
+    const int ln = threadIdx.x & (kWave - 1);
+    const int mine = ln < (int)gridDim.z ? context_lens[ln] : -0x7fffffff - 1;
+    int rank = 0;
+    for (int j = 0; j < (int)gridDim.z; ++j) {
+      const int other = __builtin_amdgcn_readlane(mine, j);
+      rank += (other > mine || (other == mine && j < ln)) ? 1 : 0;
+    }
+    const uint64_t hit = __ballot(rank == (int)blockIdx.z && ln < (int)gridDim.z);
+    b = __builtin_ctzll(hit);  // exactly one lane has each rank
+  }
   const int context_len = context_lens[b];
   const int chunk_start = split * chunk_tokens;
   if (chunk_start >= context_len) {
