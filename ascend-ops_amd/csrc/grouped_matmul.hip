@@ -110,6 +110,25 @@ __device__ __forceinline__ GmmWork gmm_find_work(const int64_t* __restrict__ gro
   return w;
 }
 
+// Scheduling directive for one k step: after every MFMA the compiler places a share of the
+// step's LDS reads (mask 0x100), LDS writes (0x200) and global loads (0x020), so that their
+// issue slots fall into the 32 cycles an MFMA (0x008) keeps the matrix core busy.
+template <int M, int NM, int NR, int NW, int NG>
+struct MfmaInterleave {
+  static __device__ __forceinline__ void run() {
+    if constexpr (M < NM) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      constexpr int r = NR * (M + 1) / NM - NR * M / NM;
+      constexpr int w = NW * (M + 1) / NM - NW * M / NM;
+      constexpr int g = NG * (M + 1) / NM - NG * M / NM;
+      if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
+      if constexpr (w > 0) __builtin_amdgcn_sched_group_barrier(0x200, w, 0);
+      if constexpr (g > 0) __builtin_amdgcn_sched_group_barrier(0x020, g, 0);
+      MfmaInterleave<M + 1, NM, NR, NW, NG>::run();
+    }
+  }
+};
+
 // LDS tile [rows][kBK] halfs, 128 bytes per row.  16-byte chunk c of row r is stored in row
 // r ^ ((r >> 3) & 1) at chunk position c ^ (r & 7): the 128-bit fragment reads of 8 or of 16
 // consecutive rows (same c) then touch every bank once, whichever width the LDS serves per
@@ -201,7 +220,7 @@ __global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
 #pragma unroll
     for (int i = 0; i < kAChunks; ++i) ra[slot][i] = ld128(a_base + kt * kBK + a_off[i]);
 #pragma unroll
-    for (int i = 0; i < kBChunks; ++i) rb[slot][i] = ld128(b_base + kt * kBK + b_off[i]);
+    for (int i = 0; i < kBChunks; ++i) rb[slot][i] = ld128_stream(b_base + kt * kBK + b_off[i]);
   };
   auto store_tile = [&](int slot, int stage) {
     f16* da = sa + stage * BM * kBK;
@@ -224,25 +243,26 @@ __global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
   const f16* sa_w = sa + wm * 32 * kBK;
   const f16* sb_w = sb + wn * 32 * NB * kBK;
 
-  // One pipeline step with LIVE live row blocks.  SLOT = register slot that holds tile kt+1,
-  // STAGE = LDS stage of tile kt.  The staging traffic (LDS writes of tile kt+1, global loads of
-  // tile kt+1+D) and the fragment reads of the next k step are issued in front of each group of
-  // MFMAs, so that they complete under the matrix cores' shadow.  Past the end of the k loop the
-  // same code runs on the last tile again (valid memory, results never consumed) instead of
-  // branching.
-  auto iteration = [&](int kt, auto slot_c, auto stage_c, auto live_c) {
-    constexpr int SLOT = decltype(slot_c)::value;
-    constexpr int STAGE = decltype(stage_c)::value;
+  // The k loop for LIVE live row blocks.  Iteration kt works on tile kt in LDS stage kt&1; the
+  // register slot (kt+1)%D holds tile kt+1.  Per iteration, four k steps of 16:
+  //   steps 0..2: MFMAs of the step | fragment reads of the next step (same stage) | a third of
+  //               the staging: LDS writes of tile kt+1 into the other stage, each followed by
+  //               the global load of tile kt+1+D into the register it just freed;
+  //   barrier   : every wave has read all its fragments of tile kt and written its part of
+  //               tile kt+1;
+  //   step 3    : MFMAs of the step | fragment reads of step 0 of tile kt+1.
+  // So the matrix cores never wait for an LDS round trip at a tile boundary, and there is one
+  // barrier per k tile.  Past the end of the k loop the same code runs on the last tile again
+  // (valid memory, results never consumed) instead of branching.
+  auto k_loop = [&](auto live_c) {
     constexpr int LIVE = decltype(live_c)::value;
-    const int kload = min(kt + 1 + D, ktiles - 1) * kBK;
-    constexpr int kAPer = (kAChunks + kSteps - 1) / kSteps;
-    constexpr int kBPer = (kBChunks + kSteps - 1) / kSteps;
-    const f16* ca = sa_w + STAGE * BM * kBK;
-    const f16* cb = sb_w + STAGE * BN * kBK;
-    f16* da = sa + (STAGE ^ 1) * BM * kBK;
-    f16* db = sb + (STAGE ^ 1) * BN * kBK;
+    constexpr int kStageSteps = kSteps - 1;  // steps that carry staging traffic
+    constexpr int kAPer = (kAChunks + kStageSteps - 1) / kStageSteps;
+    constexpr int kBPer = (kBChunks + kStageSteps - 1) / kStageSteps;
     f16x8 fa[2][LIVE > 0 ? LIVE : 1], fb[2][NB];
-    auto load_frags = [&](int buf, int st) {
+    auto load_frags = [&](int buf, int st, int stage) {
+      const f16* ca = sa_w + stage * BM * kBK;
+      const f16* cb = sb_w + stage * BN * kBK;
 #pragma unroll
       for (int j = 0; j < NB; ++j)
         fb[buf][j] = *reinterpret_cast<const f16x8*>(&cb[frag_off[st] + j * 32 * kBK]);
@@ -250,49 +270,68 @@ __global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
       for (int i = 0; i < LIVE; ++i)
         fa[buf][i] = *reinterpret_cast<const f16x8*>(&ca[frag_off[st] + i * 64 * kBK]);
     };
-    __syncthreads();  // stage STAGE is complete; stage STAGE^1 is no longer being read
-    load_frags(0, 0);
+    auto step = [&](int kload, auto slot_c, auto stage_c, auto st_c) {
+      constexpr int SLOT = decltype(slot_c)::value;
+      constexpr int STAGE = decltype(stage_c)::value;
+      constexpr int ST = decltype(st_c)::value;
+      constexpr int a_lo = ST * kAPer < kAChunks ? ST * kAPer : kAChunks;
+      constexpr int a_hi = (ST + 1) * kAPer < kAChunks ? (ST + 1) * kAPer : kAChunks;
+      constexpr int b_lo = ST * kBPer < kBChunks ? ST * kBPer : kBChunks;
+      constexpr int b_hi = (ST + 1) * kBPer < kBChunks ? (ST + 1) * kBPer : kBChunks;
+      constexpr int n_stage = ST < kStageSteps ? (a_hi - a_lo) + (b_hi - b_lo) : 0;
+      if (ST + 1 < kSteps) {
+        load_frags((ST + 1) & 1, ST + 1, STAGE);
+        f16* da = sa + (STAGE ^ 1) * BM * kBK;
+        f16* db = sb + (STAGE ^ 1) * BN * kBK;
 #pragma unroll
-    for (int st = 0; st < kSteps; ++st) {
-      if (st + 1 < kSteps) load_frags((st + 1) & 1, st + 1);
+        for (int i = a_lo; i < a_hi; ++i) {
+          *reinterpret_cast<f16x8*>(&da[st_dst + i * kRowsPerPass * kBK]) = ra[SLOT][i];
+          ra[SLOT][i] = ld128(a_base + kload + a_off[i]);
+        }
 #pragma unroll
-      for (int i = st * kAPer; i < (st + 1) * kAPer && i < kAChunks; ++i) {
-        *reinterpret_cast<f16x8*>(&da[st_dst + i * kRowsPerPass * kBK]) = ra[SLOT][i];
-        ra[SLOT][i] = ld128(a_base + kload + a_off[i]);
+        for (int i = b_lo; i < b_hi; ++i) {
+          *reinterpret_cast<f16x8*>(&db[st_dst + i * kRowsPerPass * kBK]) = rb[SLOT][i];
+          rb[SLOT][i] = ld128_stream(b_base + kload + b_off[i]);
+        }
+      } else {
+        load_frags(0, 0, STAGE ^ 1);  // first fragments of the next tile
       }
-#pragma unroll
-      for (int i = st * kBPer; i < (st + 1) * kBPer && i < kBChunks; ++i) {
-        *reinterpret_cast<f16x8*>(&db[st_dst + i * kRowsPerPass * kBK]) = rb[SLOT][i];
-        rb[SLOT][i] = ld128(b_base + kload + b_off[i]);
-      }
-      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < LIVE; ++i)
 #pragma unroll
         for (int j = 0; j < NB; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[st & 1][j], fa[st & 1][i],
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ST & 1][j], fa[ST & 1][i],
                                                              acc[i][j], 0, 0, 0);
+      MfmaInterleave<0, LIVE * NB, LIVE + NB, n_stage, n_stage>::run();
       __builtin_amdgcn_sched_barrier(0);
+    };
+    auto iteration = [&](int kt, auto slot_c, auto stage_c) {
+      const int kload = min(kt + 1 + D, ktiles - 1) * kBK;
+      step(kload, slot_c, stage_c, std::integral_constant<int, 0>{});
+      step(kload, slot_c, stage_c, std::integral_constant<int, 1>{});
+      step(kload, slot_c, stage_c, std::integral_constant<int, 2>{});
+      __syncthreads();
+      step(kload, slot_c, stage_c, std::integral_constant<int, 3>{});
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using SlotEven = std::integral_constant<int, 1 % D>;  // slot of tile kt+1 for even kt
+    using SlotOdd = std::integral_constant<int, 2 % D>;   // ... for odd kt
+    __syncthreads();  // tile 0 is in stage 0
+    load_frags(0, 0, 0);
+    int kt = 0;
+    for (; kt + 1 < ktiles; kt += 2) {
+      iteration(kt, SlotEven{}, I0{});
+      iteration(kt + 1, SlotOdd{}, I1{});
     }
+    if (kt < ktiles) iteration(kt, SlotEven{}, I0{});
   };
 
+  // tile t travels in register slot t % D and is consumed from LDS stage t & 1
   load_tile(0, 0);
   store_tile(0, 0);
 #pragma unroll
   for (int t = 1; t <= D; ++t) load_tile(t % D, min(t, ktiles - 1));
-  using I0 = std::integral_constant<int, 0>;
-  using I1 = std::integral_constant<int, 1>;
-  using SlotEven = std::integral_constant<int, 1 % D>;  // slot of tile kt+1 for even kt
-  using SlotOdd = std::integral_constant<int, 2 % D>;   // ... for odd kt
-  // tile t travels in register slot t % D and is consumed from LDS stage t & 1
-  auto k_loop = [&](auto live_c) {
-    int kt = 0;
-    for (; kt + 1 < ktiles; kt += 2) {
-      iteration(kt, SlotEven{}, I0{}, live_c);
-      iteration(kt + 1, SlotOdd{}, I1{}, live_c);
-    }
-    if (kt < ktiles) iteration(kt, SlotEven{}, I0{}, live_c);
-  };
   // One branch-free instantiation of the k loop per number of live row blocks.
   if (live >= MB) {
     k_loop(std::integral_constant<int, MB>{});
@@ -384,21 +423,17 @@ extern "C" int aops_grouped_matmul_f16(const void* x, const void* w, const int64
   const f16* wp = static_cast<const f16*>(w);
   f16* yp = static_cast<f16*>(y);
   static const int variant = [] {
-    const char* e = getenv("AOPS_GMM_VARIANT");  // tuning aid
+    const char* e = getenv("AOPS_GMM_VARIANT");  // tuning aid: tile shape / prefetch distance
     return e ? atoi(e) : 0;
   }();
   switch (variant) {
-    case 1:
+    case 1:  // 128 x 128 tiles
       return gmm_launch<2, 2, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
-    case 2:
+    case 2:  // 256 x 128 tiles
       return gmm_launch<4, 2, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
-    case 3:
+    case 3:  // 320 x 128 tiles, loads one tile ahead
       return gmm_launch<5, 2, 1>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
-    case 4:
+    default:  // 320 x 128 tiles, loads two tiles ahead
       return gmm_launch<5, 2, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
-    case 5:
-      return gmm_launch<4, 4, 1>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
-    default:
-      return gmm_launch<5, 2, 1>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
   }
 }
