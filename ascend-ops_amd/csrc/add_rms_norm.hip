@@ -39,7 +39,7 @@ __global__ __launch_bounds__(1024) void add_rms_norm_rows(const f16* __restrict_
     f16* yr = y + row * hidden;
     f16* ror = residual_out + row * hidden;
 
-    f16x8 t16[ITERS];
+    f16x8 t16[ITERS], w16[ITERS];
     float ss = 0.f;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
@@ -47,6 +47,7 @@ __global__ __launch_bounds__(1024) void add_rms_norm_rows(const f16* __restrict_
       if (v < nvec) {
         const f16x8 a = ld128_stream(xr + v * 8);
         const f16x8 b = ld128_stream(rr + v * 8);
+        w16[it] = ld128(weight + v * 8);  // in flight during the reduction
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const f16 s = (f16)((float)a[j] + (float)b[j]);  // correctly rounded fp16 add
@@ -62,10 +63,9 @@ __global__ __launch_bounds__(1024) void add_rms_norm_rows(const f16* __restrict_
     for (int it = 0; it < ITERS; ++it) {
       const int v = threadIdx.x + it * blockDim.x;
       if (v < nvec) {
-        const f16x8 w = ld128(weight + v * 8);
         f16x8 o;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) o[j] = (f16)((float)t16[it][j] * inv_rms * (float)w[j]);
+        for (int j = 0; j < 8; ++j) o[j] = (f16)((float)t16[it][j] * inv_rms * (float)w16[it][j]);
         st128_stream(yr + v * 8, o);
       }
     }

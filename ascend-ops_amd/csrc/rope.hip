@@ -32,8 +32,8 @@ __global__ __launch_bounds__(256) void rope_neox_kernel(
     dst = out_k + off;
   }
   const int64_t pos = position_ids[b];
-  const f16x8 x1 = ld128(src + c * 8);
-  const f16x8 x2 = ld128(src + half + c * 8);
+  const f16x8 x1 = ld128_stream(src + c * 8);
+  const f16x8 x2 = ld128_stream(src + half + c * 8);
   const f16x8 cs = ld128(cos_cache + pos * half + c * 8);
   const f16x8 sn = ld128(sin_cache + pos * half + c * 8);
   f16x8 o1, o2;
@@ -43,8 +43,8 @@ __global__ __launch_bounds__(256) void rope_neox_kernel(
     o1[j] = (f16)(a * cc - bb * ss);
     o2[j] = (f16)(bb * cc + a * ss);
   }
-  st128(dst + c * 8, o1);
-  st128(dst + half + c * 8, o2);
+  st128_stream(dst + c * 8, o1);
+  st128_stream(dst + half + c * 8, o2);
 }
 
 }  // namespace aops
