@@ -325,9 +325,8 @@ def paged_attention(q, key_cache, value_cache, block_tables, context_lens):
     ws_bytes = _lib.aops_paged_attention_workspace(bs, num_heads, num_kv_heads, head_dim, block_size, max_blocks)
     _check(
         ws_bytes > 0,
-        f"paged_attention: unsupported shape (head_dim={head_dim}, block_size={block_size}, "
-        f"group={num_heads // num_kv_heads}); head_dim must be 128, block_size a multiple of 32 and "
-        "num_heads/num_kv_heads one of 1, 2, 4, 8",
+        f"paged_attention: unsupported shape (head_dim={head_dim}, block_size={block_size}); "
+        "head_dim must be a multiple of 16 up to 256",
     )
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
     code = _lib.aops_paged_attention_f16(

@@ -367,18 +367,98 @@ static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t*
                                          ch.max_splits);
 }
 
-static bool pa_shape_supported(int64_t bs, int64_t num_heads, int64_t num_kv_heads,
-                               int64_t head_dim, int64_t block_size,
-                               int64_t max_blocks_per_seq) {
+// Generic path for every other shape (head_dim a multiple of 16 up to 256, any block size, any
+// whole number of query heads per kv head): one workgroup of four waves per (sequence, query
+// head); a wave takes every fourth token, its lanes split head_dim, scores are finished with a
+// wave reduction, every wave keeps its own running softmax and the four are merged through LDS.
+// Correct for all shapes the cache layout allows, not tuned: 2-byte loads.
+constexpr int kPaGenericMaxD = 256;
+
+__global__ __launch_bounds__(4 * kWave) void pa_decode_generic(
+    const f16* __restrict__ q, const f16* __restrict__ key_cache,
+    const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
+    const int32_t* __restrict__ context_lens, f16* __restrict__ out, int num_heads,
+    int num_kv_heads, int head_dim, int block_size, int max_blocks_per_seq, float scale_log2) {
+  constexpr int kPerLane = kPaGenericMaxD / kWave;
+  const int h = blockIdx.x;
+  const int b = blockIdx.y;
+  const int g = h / (num_heads / num_kv_heads);
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int context_len = context_lens[b];
+  const int64_t row_chunks = (int64_t)num_kv_heads * head_dim / 16;  // 32-byte granules per token
+  const int32_t* table = block_tables + (int64_t)b * max_blocks_per_seq;
+
+  float qf[kPerLane], acc[kPerLane];
+  int64_t elem_off[kPerLane];  // offset of (head g, dim d) inside a page, token 0
+#pragma unroll
+  for (int i = 0; i < kPerLane; ++i) {
+    const int d = lane + kWave * i;
+    const bool live = d < head_dim;
+    qf[i] = live ? (float)q[((int64_t)b * num_heads + h) * head_dim + d] : 0.f;
+    acc[i] = 0.f;
+    const int f = g * head_dim + (live ? d : 0);
+    elem_off[i] = (int64_t)(f / 16) * block_size * 16 + (f % 16);
+  }
+  float m = kNegBig, l = 0.f;
+  for (int j = wave; j < context_len; j += 4) {
+    const int blk = j / block_size;
+    const int64_t base = (int64_t)table[blk] * row_chunks * block_size * 16 +
+                         (int64_t)(j - blk * block_size) * 16;
+    float part = 0.f, vf[kPerLane];
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i) {
+      const bool live = lane + kWave * i < head_dim;
+      part += live ? qf[i] * (float)key_cache[base + elem_off[i]] : 0.f;
+      vf[i] = live ? (float)value_cache[base + elem_off[i]] : 0.f;
+    }
+    const float sc = wave_sum(part) * scale_log2;
+    const float m_new = fmaxf(m, sc);
+    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+    const float p = __builtin_amdgcn_exp2f(sc - m_new);
+    m = m_new;
+    l = l * alpha + p;
+#pragma unroll
+    for (int i = 0; i < kPerLane; ++i) acc[i] = acc[i] * alpha + p * vf[i];
+  }
+  __shared__ float sm_acc[4][kPaGenericMaxD];
+  __shared__ float sm_m[4], sm_l[4];
+#pragma unroll
+  for (int i = 0; i < kPerLane; ++i) sm_acc[wave][lane + kWave * i] = acc[i];
+  if (lane == 0) {
+    sm_m[wave] = m;
+    sm_l[wave] = l;
+  }
+  __syncthreads();
+  for (int d = threadIdx.x; d < head_dim; d += 4 * kWave) {
+    const float mx = fmaxf(fmaxf(sm_m[0], sm_m[1]), fmaxf(sm_m[2], sm_m[3]));
+    float lsum = 0.f, a = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float wt = __builtin_amdgcn_exp2f(sm_m[w] - mx);
+      lsum += sm_l[w] * wt;
+      a += sm_acc[w][d] * wt;
+    }
+    out[((int64_t)b * num_heads + h) * head_dim + d] = (f16)(lsum > 0.f ? a / lsum : 0.f);
+  }
+}
+
+static bool pa_args_valid(int64_t bs, int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                          int64_t block_size, int64_t max_blocks_per_seq) {
   if (bs < 0 || num_heads <= 0 || num_kv_heads <= 0 || max_blocks_per_seq < 0) return false;
-  if (head_dim != kPaD) return false;
-  if (block_size <= 0 || block_size % kPaStep != 0) return false;
-  if (num_heads % num_kv_heads != 0) return false;
-  const int64_t group = num_heads / num_kv_heads;
-  if (group != 1 && group != 2 && group != 4 && group != 8) return false;
-  if (bs > 65535 || num_kv_heads > 65535 || num_heads > 0x7fffffff / kPaD) return false;
+  if (head_dim <= 0 || head_dim % 16 != 0 || head_dim > kPaGenericMaxD) return false;
+  if (block_size <= 0 || num_heads % num_kv_heads != 0) return false;
+  if (bs > 65535 || num_kv_heads > 65535 || num_heads > 0x7fffffff / kPaGenericMaxD) return false;
   if (block_size * max_blocks_per_seq > 0x7fffffff) return false;
   return true;
+}
+
+// Shapes served by the MFMA kernel; everything else that is valid takes the generic kernel.
+static bool pa_fast_shape(int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                          int64_t block_size) {
+  if (head_dim != kPaD || block_size % kPaStep != 0) return false;
+  const int64_t group = num_heads / num_kv_heads;
+  return group == 1 || group == 2 || group == 4 || group == 8 || group == 16;
 }
 
 }  // namespace aops
@@ -387,8 +467,9 @@ extern "C" size_t aops_paged_attention_workspace(int64_t bs, int64_t num_heads,
                                                  int64_t num_kv_heads, int64_t head_dim,
                                                  int64_t block_size, int64_t max_blocks_per_seq) {
   using namespace aops;
-  if (!pa_shape_supported(bs, num_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq))
+  if (!pa_args_valid(bs, num_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq))
     return 0;
+  if (!pa_fast_shape(num_heads, num_kv_heads, head_dim, block_size)) return 16;  // not used
   const PaChunking ch = pa_chunking(bs, num_kv_heads, block_size, max_blocks_per_seq);
   return (size_t)bs * (size_t)num_heads * (size_t)ch.max_splits * (kPaD + 2) * sizeof(float);
 }
@@ -402,43 +483,46 @@ extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
                                         int64_t num_blocks, void* stream) {
   using namespace aops;
   (void)num_blocks;
-  if (!pa_shape_supported(bs, num_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq))
+  if (!pa_args_valid(bs, num_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq))
     return AOPS_ERR_INVALID_ARGUMENT;
   if (bs == 0) return AOPS_OK;
   if (!q || !key_cache || !value_cache || !block_tables || !context_lens || !o)
     return AOPS_ERR_INVALID_ARGUMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const f16* qp = static_cast<const f16*>(q);
+  const f16* kc = static_cast<const f16*>(key_cache);
+  const f16* vc = static_cast<const f16*>(value_cache);
+  f16* op = static_cast<f16*>(o);
+  if (!pa_fast_shape(num_heads, num_kv_heads, head_dim, block_size)) {
+    const float scale_log2 = kLog2e / __builtin_sqrtf((float)head_dim);
+    dim3 grid((unsigned)num_heads, (unsigned)bs);
+    pa_decode_generic<<<grid, 4 * kWave, 0, s>>>(qp, kc, vc, block_tables, context_lens, op,
+                                                 (int)num_heads, (int)num_kv_heads, (int)head_dim,
+                                                 (int)block_size, (int)max_blocks_per_seq,
+                                                 scale_log2);
+    return record_launch_status(hipGetLastError());
+  }
   const size_t need = aops_paged_attention_workspace(bs, num_heads, num_kv_heads, head_dim,
                                                      block_size, max_blocks_per_seq);
   if (!workspace || workspace_bytes < need) return AOPS_ERR_WORKSPACE;
   const PaChunking ch = pa_chunking(bs, num_kv_heads, block_size, max_blocks_per_seq);
   float* part_o = static_cast<float*>(workspace);
   float* part_ml = part_o + (size_t)bs * num_heads * ch.max_splits * kPaD;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const f16* qp = static_cast<const f16*>(q);
-  const f16* kc = static_cast<const f16*>(key_cache);
-  const f16* vc = static_cast<const f16*>(value_cache);
-  f16* op = static_cast<f16*>(o);
+#define AOPS_PA_CASE(G)                                                                        \
+  case G:                                                                                      \
+    pa_launch<G>(qp, kc, vc, block_tables, context_lens, op, part_o, part_ml, (int)bs,         \
+                 (int)num_heads, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq,  \
+                 ch, s);                                                                       \
+    break;
   switch (num_heads / num_kv_heads) {
-    case 1:
-      pa_launch<1>(qp, kc, vc, block_tables, context_lens, op, part_o, part_ml, (int)bs,
-                   (int)num_heads, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq, ch,
-                   s);
-      break;
-    case 2:
-      pa_launch<2>(qp, kc, vc, block_tables, context_lens, op, part_o, part_ml, (int)bs,
-                   (int)num_heads, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq, ch,
-                   s);
-      break;
-    case 4:
-      pa_launch<4>(qp, kc, vc, block_tables, context_lens, op, part_o, part_ml, (int)bs,
-                   (int)num_heads, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq, ch,
-                   s);
-      break;
+    AOPS_PA_CASE(1)
+    AOPS_PA_CASE(2)
+    AOPS_PA_CASE(4)
+    AOPS_PA_CASE(8)
+    AOPS_PA_CASE(16)
     default:
-      pa_launch<8>(qp, kc, vc, block_tables, context_lens, op, part_o, part_ml, (int)bs,
-                   (int)num_heads, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq, ch,
-                   s);
-      break;
+      return AOPS_ERR_INVALID_ARGUMENT;
   }
+#undef AOPS_PA_CASE
   return record_launch_status(hipGetLastError());
 }

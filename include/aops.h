@@ -108,8 +108,11 @@ int aops_grouped_matmul_f16(const void* x, const void* w, const int64_t* group_l
  *   o[b,h] = softmax_j( q[b,h] . K[j,g] / sqrt(head_dim) ) . V[j,g],  g = h / (num_heads/num_kv_heads)
  * The kernels split every sequence into fixed-size chunks of the KV cache and keep partial
  * results in `workspace`; aops_paged_attention_workspace() returns the bytes needed (the
- * counterpart of the reference's GetWorkspaceSize phase).  A sequence with context_len <= 0
- * gets zeros.  Block-table entries are not range-checked.
+ * counterpart of the reference's GetWorkspaceSize phase; 0 = shape not supported).  head_dim must
+ * be a multiple of 16 up to 256.  head_dim 128 with block_size a multiple of 32 and
+ * num_heads/num_kv_heads in {1, 2, 4, 8, 16} runs on the matrix cores; every other shape takes a
+ * generic, untuned kernel.  A sequence with context_len <= 0 gets zeros.  Block-table entries are
+ * not range-checked.
  * Replaces aclnnPagedAttentionExGetWorkspaceSize + aclnnPagedAttentionEx
  * (reference csrc/ffi/ops.cpp:454-461).
  */

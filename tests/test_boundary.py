@@ -62,8 +62,10 @@ def test_workspace_query_without_gpu():
     # a single short sequence is split into more chunks than a large batch
     n1 = C._lib.aops_paged_attention_workspace(1, 32, 8, 128, 128, 32)
     assert n1 // (32 * 130 * 4) > n // per_chunk
-    assert C._lib.aops_paged_attention_workspace(64, 32, 8, 96, 128, 32) == 0  # unsupported head_dim
-    assert C._lib.aops_paged_attention_workspace(64, 32, 8, 128, 24, 32) == 0  # unsupported page size
+    assert C._lib.aops_paged_attention_workspace(64, 32, 8, 100, 128, 32) == 0  # head_dim % 16 != 0
+    assert C._lib.aops_paged_attention_workspace(64, 32, 8, 512, 128, 32) == 0  # head_dim > 256
+    assert C._lib.aops_paged_attention_workspace(64, 32, 7, 128, 128, 32) == 0  # heads not a multiple of kv heads
+    assert C._lib.aops_paged_attention_workspace(64, 32, 8, 96, 24, 32) > 0     # generic kernel: token amount
 
 
 def test_c_abi_rejects_bad_sizes_without_touching_the_gpu():
@@ -80,7 +82,7 @@ def test_c_abi_rejects_bad_sizes_without_touching_the_gpu():
     assert lib.aops_reshape_and_cache_f16(None, None, None, None, None, 0, 1024, 8, 16, None) == 0
     assert lib.aops_grouped_matmul_f16(None, None, None, None, 16, 100, 2, 64, None) == -1
     assert lib.aops_grouped_matmul_f16(None, None, None, None, 0, 64, 2, 64, None) == 0
-    assert lib.aops_paged_attention_f16(None, None, None, None, None, None, None, 0, 2, 8, 2, 64, 128, 4, 16, None) == -1
+    assert lib.aops_paged_attention_f16(None, None, None, None, None, None, None, 0, 2, 8, 2, 72, 128, 4, 16, None) == -1
 
 
 H = torch.float16

@@ -269,6 +269,27 @@ def test_paged_attention(ops, dev, B, Hq, Hkv, P, lens):
     assert (o.float() - ref.float()).abs().max() < 2e-3
 
 
+@pytest.mark.parametrize(
+    "B,Hq,Hkv,D,P,lens",
+    [
+        (3, 8, 2, 64, 16, [1, 50, 200]),        # head_dim 64, small pages
+        (2, 6, 2, 128, 128, [130, 700]),        # 3 query heads per kv head
+        (2, 4, 4, 256, 32, [33, 0]),            # head_dim 256, one empty sequence
+        (2, 32, 2, 128, 64, [100, 1000]),       # 16 query heads per kv head (matrix-core path)
+        (2, 8, 2, 128, 24, [25, 300]),          # block size not a multiple of 32
+        (1, 5, 5, 48, 8, [77]),                 # head_dim 48
+    ],
+)
+def test_paged_attention_other_shapes(ops, dev, B, Hq, Hkv, D, P, lens):
+    case = _paged_case(B, Hq, Hkv, D, P, lens, seed=3, poison=True)
+    o = _run_pa(ops, dev, case)
+    ref = R.paged_attention_ref(*case)
+    assert o.shape == (B, Hq, D)
+    assert not torch.isnan(o).any()
+    torch.testing.assert_close(o.float(), ref.float(), **TOL)
+    assert (o.float() - ref.float()).abs().max() < 3e-3
+
+
 def test_paged_attention_ignores_garbage_and_unused_table_entries(ops, dev):
     lens = [5, 130, 257, 1]
     clean = _paged_case(4, 32, 8, 128, 128, lens, seed=1, max_pages=6)
