@@ -347,11 +347,11 @@ __global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
 
   // Epilogue.  acc[i][j][r]: output row 32*(wm+2i) + lane%32, output columns
   // wn*32*NB + 32j + 8*(r/4) + 4*(lane/32) + r%4.  The C tile goes to LDS as [BM][BN] halfs in
-  // 8-byte pieces, piece c of row m at position c ^ ((m & 15) << 1) (write conflicts at most
+  // 8-byte pieces, piece c of row m at position c ^ ((m & kSwz) << 1) (write conflicts at most
   // 2-way, 16-byte reads stay contiguous), and leaves as 128-bit row-contiguous global stores.
   __syncthreads();  // all waves are done with the operand stages
   f16* sc = smem;
-  constexpr int kPiecesPerRow = BN / 4;
+  constexpr int kSwz = (BN / 8 < 16 ? BN / 8 : 16) - 1;  // swizzle stays inside the row
 #pragma unroll
   for (int i = 0; i < MB; ++i) {
     const int m = 32 * (wm + 2 * i) + fm;
@@ -363,7 +363,7 @@ __global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = (f16)acc[i][j][4 * g + e];
         const int piece = (wn * 32 * NB + 32 * j + 8 * g + 4 * fq) >> 2;
-        *reinterpret_cast<f16x4*>(&sc[m * BN + ((piece ^ ((m & 15) << 1)) << 2)]) = v;
+        *reinterpret_cast<f16x4*>(&sc[m * BN + ((piece ^ ((m & kSwz) << 1)) << 2)]) = v;
       }
     }
   }
@@ -374,7 +374,7 @@ __global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
   const int col = work.n_tile * BN + c16 * 8;
   if (col < n) {
     for (int m = tid / kChunksPerRow; m < tile_rows; m += kRowsPerStorePass) {
-      const f16x8 v = *reinterpret_cast<const f16x8*>(&sc[m * BN + ((c16 ^ (m & 15)) << 3)]);
+      const f16x8 v = *reinterpret_cast<const f16x8*>(&sc[m * BN + ((c16 ^ (m & kSwz)) << 3)]);
       st128(y + (int64_t)(work.row_begin + m) * n + col, v);
     }
   }
@@ -422,18 +422,28 @@ extern "C" int aops_grouped_matmul_f16(const void* x, const void* w, const int64
   const f16* xp = static_cast<const f16*>(x);
   const f16* wp = static_cast<const f16*>(w);
   f16* yp = static_cast<f16*>(y);
-  static const int variant = [] {
-    const char* e = getenv("AOPS_GMM_VARIANT");  // tuning aid: tile shape / prefetch distance
+  static const int forced = [] {
+    const char* e = getenv("AOPS_GMM_VARIANT");  // tuning aid: 1..4 force one tile shape
     return e ? atoi(e) : 0;
   }();
+  // Tile choice from what the host knows (group_list stays on the device): the largest tile
+  // whose grid still gives every CU work.  320 rows cover a typical expert of a large routed
+  // batch in one tile; small or dense problems (few rows, one expert) take smaller tiles so that
+  // enough workgroups exist to pull the weights through all memory channels.
+  int variant = forced;
+  if (variant < 1 || variant > 4) {
+    auto tiles = [&](int64_t bm, int64_t bn) { return ((rows + bm - 1) / bm) * ((n + bn - 1) / bn); };
+    constexpr int64_t kEnough = 384;
+    variant = tiles(320, 128) >= kEnough ? 1 : tiles(256, 128) >= kEnough ? 2 : tiles(128, 128) >= kEnough ? 3 : 4;
+  }
   switch (variant) {
-    case 1:  // 128 x 128 tiles
-      return gmm_launch<2, 2, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
+    case 1:  // 320 x 128 tiles
+      return gmm_launch<5, 2, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
     case 2:  // 256 x 128 tiles
       return gmm_launch<4, 2, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
-    case 3:  // 320 x 128 tiles, loads one tile ahead
-      return gmm_launch<5, 2, 1>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
-    default:  // 320 x 128 tiles, loads two tiles ahead
-      return gmm_launch<5, 2, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
+    case 3:  // 128 x 128 tiles
+      return gmm_launch<2, 2, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
+    default:  // 64 x 64 tiles
+      return gmm_launch<1, 1, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
   }
 }
