@@ -110,15 +110,18 @@ __device__ __forceinline__ GmmWork gmm_find_work(const int64_t* __restrict__ gro
   return w;
 }
 
-// Scheduling directive for one k step: after every MFMA the compiler places a share of the
-// step's LDS reads (mask 0x100), LDS writes (0x200) and global loads (0x020), so that their
-// issue slots fall into the 32 cycles an MFMA (0x008) keeps the matrix core busy.
+// Scheduling directive for one k step.  The step's LDS fragment reads (mask 0x100) follow its
+// first two MFMAs (0x008): they feed the next step and need a full LDS round trip, so they go
+// out first.  The staging LDS writes (0x200) and global loads (0x020) are then spread over the
+// remaining MFMAs, so that their issue slots fall into the 32 cycles an MFMA keeps the matrix
+// core busy.
 template <int M, int NM, int NR, int NW, int NG>
 struct MfmaInterleave {
   static __device__ __forceinline__ void run() {
     if constexpr (M < NM) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      constexpr int r = NR * (M + 1) / NM - NR * M / NM;
+      constexpr int kReadSlots = NM < 2 ? NM : 2;
+      constexpr int r = M < kReadSlots ? NR * (M + 1) / kReadSlots - NR * M / kReadSlots : 0;
       constexpr int w = NW * (M + 1) / NM - NW * M / NM;
       constexpr int g = NG * (M + 1) / NM - NG * M / NM;
       if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
