@@ -668,7 +668,8 @@ extern "C" int aops_grouped_matmul_f16(const void* x, const void* w, const int64
   using namespace aops;
   if (rows < 0 || k <= 0 || n <= 0 || num_experts < 0 || k % 64 != 0 || n % 64 != 0)
     return AOPS_ERR_INVALID_ARGUMENT;
-  if (rows > 0x7fffffff - 4096 || k > 0x7fffffff || n > 0x7fffffff || num_experts > (1 << 20))
+  // per-lane tile offsets are 32-bit: 320 rows x k elements must fit
+  if (rows > 0x7fffffff - 4096 || k > (1 << 22) || n > 0x7fffffff || num_experts > (1 << 20))
     return AOPS_ERR_INVALID_ARGUMENT;
   if (rows == 0 || num_experts == 0) return AOPS_OK;
   if (!x || !w || !group_list || !y) return AOPS_ERR_INVALID_ARGUMENT;

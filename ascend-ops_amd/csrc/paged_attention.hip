@@ -178,9 +178,10 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
       rank += (other > mine || (other == mine && j < ln)) ? 1 : 0;
     }
     const uint64_t hit = __ballot(rank == (int)blockIdx.z && ln < (int)gridDim.z);
-    b = __builtin_ctzll(hit);  // exactly one lane has each rank
+    if (hit) b = __builtin_ctzll(hit);  // exactly one lane has each rank
   }
-  const int context_len = context_lens[b];
+  // a length beyond the block table would walk off the table row
+  const int context_len = min(context_lens[b], max_blocks_per_seq * block_size);
   const int chunk_start = split * chunk_tokens;
   if (chunk_start >= context_len) {
     if (FINAL) {  // empty sequence: zeros
@@ -385,7 +386,7 @@ __global__ __launch_bounds__(4 * kWave) void pa_decode_generic(
   const int g = h / (num_heads / num_kv_heads);
   const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x & (kWave - 1);
-  const int context_len = context_lens[b];
+  const int context_len = min(context_lens[b], max_blocks_per_seq * block_size);
   const int64_t row_chunks = (int64_t)num_kv_heads * head_dim / 16;  // 32-byte granules per token
   const int32_t* table = block_tables + (int64_t)b * max_blocks_per_seq;
 

@@ -76,7 +76,8 @@ int aops_rope_neox_f16(const void* q, const void* k, const int32_t* position_ids
  * key_cache, value_cache: [num_blocks, row_elems/16, block_size, 16];
  * slot_indices: int32 [num_tokens].  For token t with s = slot_indices[t]:
  *   cache[s / block_size, c, s % block_size, 0:16] = row[t, 16c : 16c+16]   for every c.
- * Slots outside [0, num_blocks*block_size) are skipped.  value and value_cache may both be
+ * Slots outside [0, num_blocks*block_size) are skipped; if two tokens name the same slot, which
+ * of them ends up in the cache is unspecified.  value and value_cache may both be
  * NULL (key only); if only one of them is NULL the value side is skipped.
  * Replaces aclnnReshapeAndCacheExGetWorkspaceSize + aclnnReshapeAndCacheEx
  * (reference csrc/ffi/ops.cpp:387-396).
@@ -92,7 +93,8 @@ int aops_reshape_and_cache_f16(const void* key, const void* value, void* key_cac
  * the logical [E, K, N] tensor with stride(1)==1, stride(2)==K); group_list: int64
  * [num_experts] cumulative row ends, read on the device; y: [rows, n].
  *   y[group_list[e-1] : group_list[e], :] = f16( x[...] (fp32 accumulate) @ w[e]^T )
- * Rows at or past group_list[num_experts-1] are not written.  k and n must be multiples of 64.
+ * Rows at or past group_list[num_experts-1] are not written.  k and n must be multiples of 64
+ * (k at most 2^22).
  * Replaces aclnnGroupedMatMulExGetWorkspaceSize + aclnnGroupedMatMulEx
  * (reference csrc/ffi/ops.cpp:211-218).
  */
@@ -111,8 +113,8 @@ int aops_grouped_matmul_f16(const void* x, const void* w, const int64_t* group_l
  * counterpart of the reference's GetWorkspaceSize phase; 0 = shape not supported).  head_dim must
  * be a multiple of 16 up to 256.  head_dim 128 with block_size a multiple of 32 and
  * num_heads/num_kv_heads in {1, 2, 4, 8, 16} runs on the matrix cores; every other shape takes a
- * generic, untuned kernel.  A sequence with context_len <= 0 gets zeros.  Block-table entries are
- * not range-checked.
+ * generic, untuned kernel.  A sequence with context_len <= 0 gets zeros; a context_len beyond
+ * max_blocks_per_seq*block_size is cut there.  Block-table entries are not range-checked.
  * Replaces aclnnPagedAttentionExGetWorkspaceSize + aclnnPagedAttentionEx
  * (reference csrc/ffi/ops.cpp:454-461).
  */

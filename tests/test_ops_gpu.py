@@ -110,6 +110,30 @@ def test_reshape_and_cache_reference_known_answer(ops, dev):
     assert torch.count_nonzero(vc2) == 0
 
 
+def test_reshape_and_cache_golden_fixture(ops, dev):
+    """Committed fixture (tests/golden/reshape_and_cache_kat.npz): the reference's inputs bit for
+    bit, the expected cache given as explicit flat positions."""
+    import os
+
+    import numpy as np
+
+    d = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reshape_and_cache_kat.npz"))
+    as_half = lambda a: torch.from_numpy(a.copy()).view(H)
+    key, value, key2 = as_half(d["key_bits"]), as_half(d["value_bits"]), as_half(d["key2_bits"])
+    slots = torch.from_numpy(d["slots"].copy())
+    shape = tuple(int(v) for v in d["cache_shape"])
+    idx = torch.from_numpy(d["flat_index"].reshape(-1))
+    kc = torch.zeros(shape, dtype=H, device=dev); vc = torch.zeros(shape, dtype=H, device=dev)
+    ops.reshape_and_cache(key.to(dev), value.to(dev), kc, vc, slots.to(dev))
+    want_k = torch.zeros(kc.numel(), dtype=H); want_v = torch.zeros_like(want_k)
+    want_k[idx] = key.reshape(-1); want_v[idx] = value.reshape(-1)
+    assert torch.equal(kc.cpu().reshape(-1), want_k) and torch.equal(vc.cpu().reshape(-1), want_v)
+    kc.zero_(); vc.zero_()
+    ops.reshape_and_cache(key2.to(dev), None, kc, None, slots.to(dev))  # key-only case of the reference
+    want_k.zero_(); want_k[idx] = key2.reshape(-1)
+    assert torch.equal(kc.cpu().reshape(-1), want_k) and torch.count_nonzero(vc) == 0
+
+
 @pytest.mark.parametrize("T,Hkv,D,NB,P", [(2048, 8, 128, 1024, 128), (64, 8, 128, 40, 128), (17, 2, 64, 9, 16), (5, 1, 16, 3, 7), (0, 8, 128, 4, 128)])
 def test_reshape_and_cache_bit_exact(ops, dev, T, Hkv, D, NB, P):
     g = _gen(0)

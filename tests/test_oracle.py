@@ -136,6 +136,30 @@ def test_reshape_and_cache_reference_known_answer():
     assert torch.equal(kc3, kc) and torch.count_nonzero(vc3) == 0
 
 
+def _load_kat():
+    import os
+    d = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reshape_and_cache_kat.npz"))
+    as_half = lambda a: torch.from_numpy(a.copy()).view(torch.float16)
+    return d, as_half(d["key_bits"]), as_half(d["value_bits"]), as_half(d["key2_bits"]), torch.from_numpy(d["slots"].copy())
+
+
+def test_reshape_and_cache_golden_fixture():
+    """The committed fixture of the reference's known-answer case: inputs bit for bit, expected
+    positions as explicit flat indices (tests/golden/make_reshape_and_cache_kat.py)."""
+    d, key, value, key2, slots = _load_kat()
+    assert d["blocks"].tolist() == [0, 1, 1, 2] and d["offsets"].tolist() == [6, 6, 84, 34]
+    # the fixture's inputs are what the reference's seed produces today
+    torch.manual_seed(42)
+    assert torch.equal(torch.randn(4, 8, 128, dtype=torch.float16), key)
+    shape = tuple(int(v) for v in d["cache_shape"])
+    kc = torch.zeros(shape, dtype=torch.float16); vc = torch.zeros_like(kc)
+    R.reshape_and_cache_ref(key, kc, slots, value, vc)
+    want_k = torch.zeros(kc.numel(), dtype=torch.float16); want_v = torch.zeros_like(want_k)
+    idx = torch.from_numpy(d["flat_index"].reshape(-1))
+    want_k[idx] = key.reshape(-1); want_v[idx] = value.reshape(-1)
+    assert torch.equal(kc.reshape(-1), want_k) and torch.equal(vc.reshape(-1), want_v)
+
+
 def test_reshape_and_cache_pack_roundtrip_and_skips():
     torch.manual_seed(4)
     NB, P, H, D = 3, 32, 2, 64
