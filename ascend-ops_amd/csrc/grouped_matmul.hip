@@ -607,6 +607,431 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
   }
 }
 
+// Per-lane summary of group_list for workgroups that look up many work items: lane l covers
+// experts [l*per, (l+1)*per).
+constexpr int kBndCache = 4;
+struct GmmPlan {
+  int per;          // experts per lane
+  int tiles;        // m-tiles of this lane's experts
+  int incl;         // inclusive prefix of tiles over the lanes
+  int total_tiles;  // over all experts
+  int bnd[kBndCache + 1];  // clamped row ends of experts l*per-1 .. l*per+kBndCache-1 (per <= kBndCache)
+};
+
+template <int kBM>
+__device__ __forceinline__ GmmPlan gmm_make_plan(const int64_t* __restrict__ group_list,
+                                                 int num_experts, int64_t rows) {
+  const int lane = threadIdx.x & (kWave - 1);
+  auto clampr = [&](int64_t v) -> int { return (int)(v < 0 ? 0 : (v > rows ? rows : v)); };
+  GmmPlan p;
+  p.per = (num_experts + kWave - 1) / kWave;
+  const int e0 = lane * p.per;
+  int prev = (e0 == 0 || e0 > num_experts) ? 0 : clampr(group_list[e0 - 1]);
+  p.bnd[0] = prev;
+  p.tiles = 0;
+  if (p.per <= kBndCache) {
+#pragma unroll
+    for (int j = 0; j < kBndCache; ++j) {
+      const int e = e0 + j;
+      int end = prev;  // slots past the lane's experts: empty
+      if (j < p.per && e < num_experts) {
+        end = clampr(group_list[e]);
+        if (end > prev) p.tiles += (end - prev + kBM - 1) / kBM;
+      }
+      p.bnd[j + 1] = end;
+      prev = end;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < kBndCache; ++j) p.bnd[j + 1] = 0;
+    for (int j = 0; j < p.per; ++j) {
+      const int e = e0 + j;
+      if (e < num_experts) {
+        const int end = clampr(group_list[e]);
+        if (end > prev) p.tiles += (end - prev + kBM - 1) / kBM;
+        prev = end;
+      }
+    }
+  }
+  int incl = p.tiles;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int up = __shfl_up(incl, d);
+    if (lane >= d) incl += up;
+  }
+  p.incl = incl;
+  p.total_tiles = __shfl(incl, kWave - 1);
+  return p;
+}
+
+// Work item `work` (0 <= work < total_tiles * n_tiles) -> (expert, m-tile, n-tile); the m-tiles
+// that share a weight tile are adjacent.  With at most kBndCache experts per lane nothing is
+// read from memory.
+template <int kBM>
+__device__ __forceinline__ GmmWork gmm_locate(const GmmPlan& p,
+                                              const int64_t* __restrict__ group_list,
+                                              int num_experts, int64_t rows, int n_tiles,
+                                              int64_t work) {
+  const int lane = threadIdx.x & (kWave - 1);
+  auto clampr = [&](int64_t v) -> int { return (int)(v < 0 ? 0 : (v > rows ? rows : v)); };
+  const int64_t lo = (int64_t)(p.incl - p.tiles) * n_tiles;
+  const int64_t hi = (int64_t)p.incl * n_tiles;
+  const bool mine = work >= lo && work < hi;
+  int f_expert = 0, f_begin = 0, f_end = 0, f_ntile = 0;
+  if (mine) {
+    const int e0 = lane * p.per;
+    int64_t base = lo;
+    if (p.per <= kBndCache) {
+      int prev = p.bnd[0];
+      bool found = false;
+#pragma unroll
+      for (int j = 0; j < kBndCache; ++j) {
+        const int end = p.bnd[j + 1];
+        const int t = (j < p.per && end > prev) ? (end - prev + kBM - 1) / kBM : 0;
+        const int64_t span = (int64_t)t * n_tiles;
+        if (!found && t > 0 && work < base + span) {
+          const int local = (int)(work - base);
+          f_expert = e0 + j;
+          f_ntile = local / t;
+          f_begin = prev + (local - f_ntile * t) * kBM;
+          f_end = end;
+          found = true;
+        }
+        base += span;
+        prev = end;
+      }
+    } else {
+      int prev = (e0 == 0) ? 0 : clampr(group_list[e0 - 1]);
+      for (int j = 0; j < p.per; ++j) {
+        const int e = e0 + j;
+        if (e >= num_experts) break;
+        const int end = clampr(group_list[e]);
+        const int t = end > prev ? (end - prev + kBM - 1) / kBM : 0;
+        const int64_t span = (int64_t)t * n_tiles;
+        if (work < base + span) {
+          const int local = (int)(work - base);
+          f_expert = e;
+          f_ntile = local / t;
+          f_begin = prev + (local - f_ntile * t) * kBM;
+          f_end = end;
+          break;
+        }
+        base += span;
+        prev = end;
+      }
+    }
+  }
+  const uint64_t mask = __ballot(mine);
+  GmmWork w;
+  w.valid = mask != 0;
+  const int src = w.valid ? __builtin_ctzll(mask) : 0;
+  w.expert = __builtin_amdgcn_readfirstlane(__shfl(f_expert, src));
+  w.row_begin = __builtin_amdgcn_readfirstlane(__shfl(f_begin, src));
+  w.row_end = __builtin_amdgcn_readfirstlane(__shfl(f_end, src));
+  w.n_tile = __builtin_amdgcn_readfirstlane(__shfl(f_ntile, src));
+  return w;
+}
+
+// Persistent form of grouped_matmul_dma_kernel: one workgroup per CU walks through its share of
+// the work items (XCD x owns a contiguous range of items, its workgroups take them round robin),
+// and the operand pipeline never drains between items: the last two k tiles of an item issue the
+// copies of the first two tiles of the next item, and the finished accumulators leave straight
+// from registers (lane pairs exchange halves with v_permlane32_swap so that every lane stores 16
+// contiguous bytes) while those copies are in flight, with no LDS use and no workgroup barrier.
+// group_list is scanned once per workgroup; every wave keeps its copy of the scan in LDS.
+// Requires k % 128 == 0 and k >= 256 (an even number of k tiles keeps the stage parity fixed).
+template <int MB, int NB, int WN>
+__global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kernel(
+    const f16* __restrict__ x, const f16* __restrict__ w, const int64_t* __restrict__ group_list,
+    f16* __restrict__ y, int64_t rows, int k, int num_experts, int n) {
+  constexpr int kWaves = 2 * WN;
+  constexpr int BM = 64 * MB;
+  constexpr int BN = 32 * NB * WN;
+  constexpr int kSteps = kBK / 16;
+  constexpr int kACopies = BM / 8 / kWaves;
+  constexpr int kBCopies = BN / 8 / kWaves;
+  static_assert(BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0, "tile rows per copy");
+
+  extern __shared__ __attribute__((aligned(16))) f16 smem[];
+  f16* sa = smem;                         // [2][BM * kBK]
+  f16* sb = smem + 2 * BM * kBK;          // [2][BN * kBK]
+  int* splan = reinterpret_cast<int*>(smem + 2 * (BM + BN) * kBK);  // [kWaves][kWave][8]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave / WN;
+  const int wn = wave % WN;
+  const int n_tiles = (n + BN - 1) / BN;
+  const int ktiles = k / kBK;
+
+  int* my_plan = splan + (wave * kWave + lane) * 8;
+  int plan_per, plan_total;
+  {
+    const GmmPlan plan = gmm_make_plan<BM>(group_list, num_experts, rows);
+    plan_per = __builtin_amdgcn_readfirstlane(plan.per);
+    plan_total = __builtin_amdgcn_readfirstlane(plan.total_tiles);
+    my_plan[0] = plan.tiles;
+    my_plan[1] = plan.incl;
+#pragma unroll
+    for (int j = 0; j <= kBndCache; ++j) my_plan[2 + j] = plan.bnd[j];
+  }
+  const int64_t total_work = (int64_t)plan_total * n_tiles;
+  const int64_t share = (total_work + kXcds - 1) / kXcds;
+  const int xcd = blockIdx.x % kXcds;
+  const int wg_in_xcd = blockIdx.x / kXcds;
+  const int wgs_per_xcd = gridDim.x / kXcds;
+  auto locate = [&](int64_t local) -> GmmWork {
+    const int64_t item = (int64_t)xcd * share + local;
+    if (local >= share || item >= total_work) {
+      GmmWork none;
+      none.valid = false;
+      none.expert = none.row_begin = none.row_end = none.n_tile = 0;
+      return none;
+    }
+    GmmPlan plan;  // this lane's part, written by this lane: no synchronisation needed
+    plan.per = plan_per;
+    plan.total_tiles = plan_total;
+    plan.tiles = my_plan[0];
+    plan.incl = my_plan[1];
+#pragma unroll
+    for (int j = 0; j <= kBndCache; ++j) plan.bnd[j] = my_plan[2 + j];
+    return gmm_locate<BM>(plan, group_list, num_experts, rows, n_tiles, item);
+  };
+
+  int64_t local = wg_in_xcd;
+  GmmWork cur = locate(local);
+  if (!cur.valid) return;
+
+  // Copy sources of the item whose tiles are being fetched.  Copy i of this wave fills physical
+  // rows (kWaves*i + wave)*8 .. +7 of a stage, i.e. logical row 8*kWaves*i + lane_row (the row
+  // swizzle only swaps rows inside the 8-row group) and chunk lane_c: one per-lane offset plus a
+  // uniform stride per copy, clamped to the last valid row: tile rows past the end of the group
+  // (only dead output rows depend on them) and past the end of w repeat the last valid row, which
+  // costs one cache line per copy instead of eight.
+  const f16* a_base;
+  const f16* b_base;
+  const int lane_row = wave * 8 + ((lane >> 3) ^ (wave & 1));
+  const int lane_c = (lane & 7) ^ (lane_row & 7);
+  const uint32_t off0 = (uint32_t)lane_row * (uint32_t)k + lane_c * 8;
+  const uint32_t copy_stride = 8u * kWaves * (uint32_t)k;
+  uint32_t a_last, b_last;  // offset of this lane's chunk in the last valid row
+  auto set_sources = [&](const GmmWork& it) {
+    a_base = x + (int64_t)it.row_begin * k;
+    b_base = w + ((int64_t)it.expert * n + (int64_t)it.n_tile * BN) * k;
+    const int n_left = min(n - it.n_tile * BN, BN);
+    const int x_left = min(it.row_end - it.row_begin, BM);  // rows of the group in this tile
+    a_last = (uint32_t)(x_left - 1) * (uint32_t)k + lane_c * 8;
+    b_last = (uint32_t)(n_left - 1) * (uint32_t)k + lane_c * 8;
+  };
+  auto copy_tile = [&](int kt, int stage) {
+    const int ko = kt * kBK;
+    f16* da = sa + stage * BM * kBK + wave * 512;
+    f16* db = sb + stage * BN * kBK + wave * 512;
+#pragma unroll
+    for (int i = 0; i < kACopies; ++i)
+      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(a_base + ko + min(off0 + i * copy_stride, a_last)),
+                                       AOPS_LDS_PTR(da + i * kWaves * 512), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < kBCopies; ++i)
+      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(b_base + ko + min(off0 + i * copy_stride, b_last)),
+                                       AOPS_LDS_PTR(db + i * kWaves * 512), 16, 0, 0);
+  };
+
+  const int fm = lane & 31;
+  const int fq = lane >> 5;
+  // Fragment addresses: lds_off(fm, 2*st + fq) == lds_off(fm, fq) ^ (st << 4) (the k step only
+  // flips two chunk bits), so one per-lane offset per operand serves every k step.
+  const int fa_off0 = lds_off(fm, fq) + wm * 32 * kBK;
+  const int fb_off0 = lds_off(fm, fq) + wn * 32 * NB * kBK;
+
+  f32x16 acc[MB][NB];
+  GmmWork nxt;
+
+  auto k_loop = [&](auto live_c) {
+    constexpr int LIVE = decltype(live_c)::value;
+    f16x8 fa[2][LIVE > 0 ? LIVE : 1], fb[2][NB];
+    auto load_frags = [&](int buf, int st, int stage) {
+      // the empty asm keeps the compiler from hoisting one address register per (stage, step)
+      // out of the k loop, which would push the accumulators into scratch
+      int fo_a = fa_off0, fo_b = fb_off0;
+      asm volatile("" : "+v"(fo_a), "+v"(fo_b));
+      const f16* ca = sa + stage * BM * kBK + (fo_a ^ (st << 4));
+      const f16* cb = sb + stage * BN * kBK + (fo_b ^ (st << 4));
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        fb[buf][j] = *reinterpret_cast<const f16x8*>(&cb[j * 32 * kBK]);
+#pragma unroll
+      for (int i = 0; i < LIVE; ++i)
+        fa[buf][i] = *reinterpret_cast<const f16x8*>(&ca[i * 64 * kBK]);
+    };
+    auto step = [&](int kcopy, auto stage_c, auto st_c) {
+      constexpr int STAGE = decltype(stage_c)::value;
+      constexpr int ST = decltype(st_c)::value;
+      if (ST + 1 < kSteps) {
+        load_frags((ST + 1) & 1, ST + 1, STAGE);
+      } else {
+        load_frags(0, 0, STAGE ^ 1);  // first fragments of the next tile
+        copy_tile(kcopy, STAGE);      // this stage is free: everyone is past the barrier
+      }
+#pragma unroll
+      for (int i = 0; i < LIVE; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ST & 1][j], fa[ST & 1][i],
+                                                             acc[i][j], 0, 0, 0);
+      MfmaInterleave<0, LIVE * NB, LIVE + NB, 0,
+                     (ST + 1 < kSteps) ? 0 : kACopies + kBCopies>::run();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto iteration = [&](int kcopy, auto stage_c) {
+      step(kcopy, stage_c, std::integral_constant<int, 0>{});
+      step(kcopy, stage_c, std::integral_constant<int, 1>{});
+      step(kcopy, stage_c, std::integral_constant<int, 2>{});
+      // own copies of the next tile and all own fragment reads of this tile are complete ...
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();  // ... and so are everybody else's
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      step(kcopy, stage_c, std::integral_constant<int, 3>{});
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    load_frags(0, 0, 0);
+    for (int kt = 0; kt < ktiles; kt += 2) {
+      int c0 = kt + 2, c1 = kt + 3;
+      if (kt + 2 >= ktiles) {  // the last two tiles fetch the head of the next item
+        if (nxt.valid) {
+          set_sources(nxt);
+          c0 = 0;
+          c1 = 1;
+        } else {  // nothing follows: repeat the last tile (valid memory, never consumed)
+          c0 = c1 = ktiles - 1;
+        }
+      }
+      iteration(c0, I0{});
+      iteration(c1, I1{});
+    }
+  };
+
+  set_sources(cur);
+  copy_tile(0, 0);
+  copy_tile(1, 1);
+  // tile 0 must be complete, tile 1 may still be on its way
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kACopies + kBCopies));
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+
+  for (;;) {
+    local += wgs_per_xcd;
+    nxt = locate(local);
+    const int tile_rows = min(cur.row_end - cur.row_begin, BM);
+    const int live_blocks = (tile_rows + 31) / 32;
+    const int live = (live_blocks - wm + 1) / 2;
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    if (live >= MB) {
+      k_loop(std::integral_constant<int, MB>{});
+    } else if (MB > 1 && live == MB - 1) {
+      k_loop(std::integral_constant<int, (MB > 1 ? MB - 1 : 0)>{});
+    } else if (MB > 2 && live == MB - 2) {
+      k_loop(std::integral_constant<int, (MB > 2 ? MB - 2 : 0)>{});
+    } else if (live >= 1) {
+      k_loop(std::integral_constant<int, (MB > 3 ? MB - 3 : 1)>{});
+    } else {
+      k_loop(std::integral_constant<int, 0>{});
+    }
+
+    // Epilogue of `cur`.  acc[i][j][4g+e]: output row 32*(wm+2i) + fm, output column
+    // wn*32*NB + 32j + 8g + 4fq + e.  For a pair of column groups (g, g+1) the two lanes of a row
+    // (fq = 0, 1) exchange halves: v_permlane32_swap trades the upper 32 lanes of its first
+    // operand for the lower 32 lanes of its second, after which lane fq holds the 8 consecutive
+    // columns of group g+fq.
+    const int col_w = cur.n_tile * BN + wn * 32 * NB;
+    const int m_w = 32 * wm + fm;
+#pragma unroll
+    for (int i = 0; i < MB; ++i) {
+      const int m = m_w + 64 * i;
+      if (i < live) {  // wave uniform: both lanes of every pair take part in the exchange
+        const bool row_ok = m < tile_rows;
+        f16* yrow = y + (int64_t)(cur.row_begin + m) * n + col_w + 8 * fq;
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+          if (col_w + 32 * j < n) {
+#pragma unroll
+            for (int gp = 0; gp < 2; ++gp) {
+              f16x4 p0, p1;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                p0[e] = (f16)acc[i][j][8 * gp + e];
+                p1[e] = (f16)acc[i][j][8 * gp + 4 + e];
+              }
+              const u32x2 d0 = __builtin_bit_cast(u32x2, p0);
+              const u32x2 d1 = __builtin_bit_cast(u32x2, p1);
+              const auto lo = __builtin_amdgcn_permlane32_swap(d0[0], d1[0], false, false);
+              const auto hi = __builtin_amdgcn_permlane32_swap(d0[1], d1[1], false, false);
+              u32x4 out;
+              out[0] = lo[0];
+              out[1] = hi[0];
+              out[2] = lo[1];
+              out[3] = hi[1];
+              if (row_ok) st128(yrow + 32 * j + 16 * gp, __builtin_bit_cast(f16x8, out));
+            }
+          }
+        }
+      }
+    }
+    if (!nxt.valid) break;
+    cur = nxt;
+  }
+  // the repeated last-tile copies must have landed before the LDS is released
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+}
+
+template <int MB, int NB, int WN>
+static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* group_list, f16* y,
+                                 int64_t rows, int k, int num_experts, int n, hipStream_t stream) {
+  constexpr int BM = 64 * MB;
+  constexpr int BN = 32 * NB * WN;
+  constexpr int kWaves = 2 * WN;
+  constexpr int kLds = 2 * (BM + BN) * kBK * (int)sizeof(f16) + kWaves * kWave * 8 * (int)sizeof(int);
+  static_assert(kLds <= 160 * 1024, "LDS budget");
+  static int cus[64] = {0};  // per device; benign race: every writer stores the same value
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return record_launch_status(e);
+  if (dev < 0 || dev >= 64) return AOPS_ERR_INVALID_ARGUMENT;
+  if (cus[dev] == 0) {
+    int v = 0;
+    e = hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return record_launch_status(e);
+    cus[dev] = v > 0 ? v : 8;
+  }
+  const int64_t n_tiles = (n + BN - 1) / BN;
+  const int64_t max_work = ((rows + BM - 1) / BM + num_experts) * n_tiles;
+  int64_t grid = cus[dev] < max_work ? cus[dev] : max_work;
+  grid = grid / kXcds * kXcds;
+  if (grid < kXcds) grid = kXcds;
+  auto kernel = grouped_matmul_persistent_kernel<MB, NB, WN>;
+  static bool attr_set = false;  // benign race: the call is idempotent
+  if (!attr_set) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return record_launch_status(e);
+    attr_set = true;
+  }
+  kernel<<<(unsigned)grid, 2 * WN * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts,
+                                                          n);
+  return record_launch_status(hipGetLastError());
+}
+
 template <int MB, int NB, int WN>
 static int gmm_dma_launch(const f16* x, const f16* w, const int64_t* group_list, f16* y,
                           int64_t rows, int k, int num_experts, int n, hipStream_t stream) {
@@ -677,22 +1102,24 @@ extern "C" int aops_grouped_matmul_f16(const void* x, const void* w, const int64
   const f16* xp = static_cast<const f16*>(x);
   const f16* wp = static_cast<const f16*>(w);
   f16* yp = static_cast<f16*>(y);
-  static const int forced = [] {
-    const char* e = getenv("AOPS_GMM_VARIANT");  // tuning aid: 1..5 force one tile shape
-    return e ? atoi(e) : 0;
-  }();
+  const char* forced_env = getenv("AOPS_GMM_VARIANT");  // tuning aid: 1..6 force one kernel / tile shape
+  const int forced = forced_env ? atoi(forced_env) : 0;
   // Tile choice from what the host knows (group_list stays on the device): the largest tile
   // whose grid still gives every CU work.  320 rows cover a typical expert of a large routed
   // batch in one tile; small or dense problems (few rows, one expert) take smaller tiles so that
   // enough workgroups exist to pull the weights through all memory channels.
   int variant = forced;
-  if (variant < 1 || variant > 5) {
+  if (variant < 1 || variant > 6) {
     auto tiles = [&](int64_t bm, int64_t bn) { return ((rows + bm - 1) / bm) * ((n + bn - 1) / bn); };
     constexpr int64_t kEnough = 384;
-    variant = tiles(320, 256) >= kEnough ? 1 : tiles(320, 128) >= kEnough ? 2 : tiles(256, 128) >= kEnough ? 3
+    variant = tiles(320, 256) >= kEnough ? 6 : tiles(320, 128) >= kEnough ? 2 : tiles(256, 128) >= kEnough ? 3
               : tiles(128, 128) >= kEnough ? 4 : 5;
   }
+  if (variant == 6 && (k % 128 != 0 || k < 256)) variant = 1;  // the persistent kernel's k loop
   switch (variant) {
+    case 6:  // 320 x 256 tiles, eight waves, one persistent workgroup per CU
+      return gmm_persistent_launch<5, 2, 4>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts,
+                                            (int)n, s);
     case 1:  // 320 x 256 tiles, eight waves, operands copied HBM -> LDS directly
       return gmm_dma_launch<5, 2, 4>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n,
                                      s);

@@ -229,6 +229,33 @@ def test_grouped_matmul_does_not_write_past_the_last_group(ops, dev):
     torch.testing.assert_close(y.cpu()[:110].float(), ref[:110].float(), **GMM_TOL)
 
 
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize(
+    "rows,K,N,E,counts",
+    [
+        (1300, 256, 192, 6, [0, 1, 700, 0, 330, 200]),   # empty groups, one row, 3-tile and 2-tile groups, 69 rows unrouted
+        (2500, 384, 576, 300, None),                      # more experts than the per-lane cache of the scan covers
+        (4096, 512, 2048, 64, None),                      # several work items per workgroup of the persistent kernel
+        (321, 256, 64, 1, [321]),                         # one expert, one row past a full tile, minimum N
+    ],
+)
+def test_grouped_matmul_every_kernel(ops, dev, monkeypatch, variant, rows, K, N, E, counts):
+    """The tile shape / kernel is normally chosen from the problem size; AOPS_GMM_VARIANT forces one,
+    so that every kernel sees the edge cases (6 = persistent kernel, needs K % 128 == 0, K >= 256)."""
+    import ascend910a_extras.ascend910a_extras_C as C
+    monkeypatch.setenv("AOPS_GMM_VARIANT", str(variant))
+    x, w, gl = _gmm_case(rows, K, N, E, seed=variant, counts=counts)
+    end = int(gl[-1])
+    y = torch.full((rows, N), 5.0, dtype=H, device=dev)
+    xd, wd, gd = x.to(dev), w.transpose(1, 2).contiguous().to(dev), gl.to(dev)   # storage [E, N, K]
+    code = C._lib.aops_grouped_matmul_f16(xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y.data_ptr(), rows, K, E, N,
+                                          torch.cuda.current_stream().cuda_stream)
+    assert code == 0
+    ref = R.grouped_matmul_ref(x, w, gl)
+    torch.testing.assert_close(y.cpu()[:end].float(), ref[:end].float(), **GMM_TOL)
+    assert torch.all(y[end:] == 5.0)
+
+
 def test_dense_mlp_chain(ops, dev):
     """benchmark/test_mlp.py:37-41 through grouped_matmul with one expert (reduced width)."""
     g = _gen(0)
