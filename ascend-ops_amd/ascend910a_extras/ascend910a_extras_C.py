@@ -33,6 +33,7 @@ _SIGNATURES = {
     "aops_rope_neox_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_reshape_and_cache_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_grouped_matmul_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "aops_grouped_matmul_swiglu_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_paged_attention_workspace": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64]),
     "aops_paged_attention_f16": (
         ctypes.c_int,
@@ -154,47 +155,71 @@ def swiglu(x):
     return y
 
 
-def grouped_matmul(x, w, group_list):
-    """reference csrc/ffi/ops.cpp:157-233."""
+def _check_grouped_matmul(name, x, w, group_list):
+    """Argument checks of reference csrc/ffi/ops.cpp:158-174 plus dtype, device and packing."""
     _check(
         x.dim() == 2 and w.dim() == 3 and group_list.dim() == 1,
-        "grouped_matmul: input tensors must be 2D and group_list must be 1D",
+        f"{name}: input tensors must be 2D and group_list must be 1D",
     )
-    num_tokens, dim = x.shape
+    dim = x.size(1)
     num_experts, inner_dim = w.size(0), w.size(2)
     _check(
         dim == w.size(1),
-        f"grouped_matmul: last dimension of x must match second dimension of w, got {dim} and {w.size(1)}",
+        f"{name}: last dimension of x must match second dimension of w, got {dim} and {w.size(1)}",
     )
     _check(
         x.is_contiguous() and group_list.is_contiguous(),
-        "grouped_matmul: x and group_list must be contiguous tensors",
+        f"{name}: x and group_list must be contiguous tensors",
     )
     _check(
         w.stride(1) == 1 and w.stride(2) == dim,
-        f"grouped_matmul: w must be K-major order, got strides {tuple(w.stride())}",
+        f"{name}: w must be K-major order, got strides {tuple(w.stride())}",
     )
     _check(
         w.size(1) % 64 == 0 and w.size(2) % 64 == 0,
-        f"grouped_matmul: second and third dimensions of w must be multiples of 64, got {w.size(1)} and {w.size(2)}",
+        f"{name}: second and third dimensions of w must be multiples of 64, got {w.size(1)} and {w.size(2)}",
     )
     _check(
         num_experts <= 1 or w.stride(0) == dim * inner_dim,
-        f"grouped_matmul: experts of w must be densely packed, got strides {tuple(w.stride())}",
+        f"{name}: experts of w must be densely packed, got strides {tuple(w.stride())}",
     )
     _check(
         group_list.size(0) == num_experts,
-        f"grouped_matmul: group_list must have one entry per expert, got {group_list.size(0)} and {num_experts}",
+        f"{name}: group_list must have one entry per expert, got {group_list.size(0)} and {num_experts}",
     )
     _require_device(
-        "grouped_matmul",
+        name,
         {"x": (x, torch.float16), "w": (w, torch.float16), "group_list": (group_list, torch.int64)},
     )
+
+
+def grouped_matmul(x, w, group_list):
+    """reference csrc/ffi/ops.cpp:157-233."""
+    _check_grouped_matmul("grouped_matmul", x, w, group_list)
+    num_tokens, dim = x.shape
+    num_experts, inner_dim = w.size(0), w.size(2)
     y = torch.empty((num_tokens, inner_dim), dtype=x.dtype, device=x.device)
     code = _lib.aops_grouped_matmul_f16(
         _ptr(x), _ptr(w), _ptr(group_list), _ptr(y), num_tokens, dim, num_experts, inner_dim, _stream(x.device)
     )
     _status("grouped_matmul", code)
+    return y
+
+
+def grouped_matmul_swiglu(x, w, group_list):
+    """swiglu(grouped_matmul(x, w, group_list)) in one kernel where the fused kernel supports the
+    shape (K a multiple of 128, at least 256), as two kernels otherwise.  Not part of the
+    reference's surface: it fuses the chain csrc/ffi/ops.cpp:157-233 -> 110-154 of an expert MLP."""
+    _check_grouped_matmul("grouped_matmul_swiglu", x, w, group_list)
+    num_tokens, dim = x.shape
+    num_experts, inner_dim = w.size(0), w.size(2)
+    if dim % 128 != 0 or dim < 256:
+        return swiglu(grouped_matmul(x, w, group_list))
+    y = torch.empty((num_tokens, inner_dim // 2), dtype=x.dtype, device=x.device)
+    code = _lib.aops_grouped_matmul_swiglu_f16(
+        _ptr(x), _ptr(w), _ptr(group_list), _ptr(y), num_tokens, dim, num_experts, inner_dim, _stream(x.device)
+    )
+    _status("grouped_matmul_swiglu", code)
     return y
 
 

@@ -740,7 +740,14 @@ __device__ __forceinline__ GmmWork gmm_locate(const GmmPlan& p,
 // contiguous bytes) while those copies are in flight, with no LDS use and no workgroup barrier.
 // group_list is scanned once per workgroup; every wave keeps its copy of the scan in LDS.
 // Requires k % 128 == 0 and k >= 256 (an even number of k tiles keeps the stage parity fixed).
-template <int MB, int NB, int WN>
+//
+// SWIGLU = true fuses the activation of a gate_up projection into the epilogue: with d = n/2 the
+// kernel writes y[r, c] = silu(h[r, c]) * h[r, d + c] (h = x @ W_e^T in fp32, never stored) as a
+// [rows, d] matrix.  A work item then covers 32*WN output columns; the weight stage holds, for wave
+// column wn, the 32 gate rows of its columns in row block 2*wn and the matching 32 up rows in row
+// block 2*wn + 1, so that a lane finds gate and up value of one output element in acc[i][0] and
+// acc[i][1].
+template <int MB, int NB, int WN, bool SWIGLU>
 __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kernel(
     const f16* __restrict__ x, const f16* __restrict__ w, const int64_t* __restrict__ group_list,
     f16* __restrict__ y, int64_t rows, int k, int num_experts, int n) {
@@ -751,6 +758,9 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   constexpr int kACopies = BM / 8 / kWaves;
   constexpr int kBCopies = BN / 8 / kWaves;
   static_assert(BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0, "tile rows per copy");
+  static_assert(!SWIGLU || (NB == 2 && kWaves == 8), "gate/up pairing assumes 64-row copies, two column blocks");
+  constexpr int BNO = SWIGLU ? BN / 2 : BN;  // output columns per work item
+  const int n_out = SWIGLU ? n / 2 : n;      // output row length
 
   extern __shared__ __attribute__((aligned(16))) f16 smem[];
   f16* sa = smem;                         // [2][BM * kBK]
@@ -762,7 +772,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int wm = wave / WN;
   const int wn = wave % WN;
-  const int n_tiles = (n + BN - 1) / BN;
+  const int n_tiles = (n_out + BNO - 1) / BNO;
   const int ktiles = k / kBK;
 
   int* my_plan = splan + (wave * kWave + lane) * 8;
@@ -816,13 +826,25 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   const uint32_t off0 = (uint32_t)lane_row * (uint32_t)k + lane_c * 8;
   const uint32_t copy_stride = 8u * kWaves * (uint32_t)k;
   uint32_t a_last, b_last;  // offset of this lane's chunk in the last valid row
+  // SWIGLU: copy i of the weights fills row blocks 2i (gate rows 32i..32i+31 of the item) and
+  // 2i+1 (the up rows d further down): per-lane offset + 32 rows per copy; b_last then holds the
+  // number of valid 32-column blocks of the item instead of an offset.
+  const uint32_t off0_glu = ((uint32_t)(lane_row & 31) + (lane_row >= 32 ? (uint32_t)n_out : 0u)) * (uint32_t)k + lane_c * 8;
   auto set_sources = [&](const GmmWork& it) {
     a_base = x + (int64_t)it.row_begin * k;
-    b_base = w + ((int64_t)it.expert * n + (int64_t)it.n_tile * BN) * k;
-    const int n_left = min(n - it.n_tile * BN, BN);
+    b_base = w + ((int64_t)it.expert * n + (int64_t)it.n_tile * BNO) * k;
+    const int n_left = min(n_out - it.n_tile * BNO, BNO);
     const int x_left = min(it.row_end - it.row_begin, BM);  // rows of the group in this tile
     a_last = (uint32_t)(x_left - 1) * (uint32_t)k + lane_c * 8;
-    b_last = (uint32_t)(n_left - 1) * (uint32_t)k + lane_c * 8;
+    b_last = SWIGLU ? (uint32_t)(n_left / 32) : (uint32_t)(n_left - 1) * (uint32_t)k + lane_c * 8;
+  };
+  auto b_offset = [&](int i) -> uint32_t {
+    if constexpr (SWIGLU) {
+      const uint32_t blk = (uint32_t)i < b_last ? (uint32_t)i : 0u;  // blocks past n: repeat block 0
+      return off0_glu + blk * 32u * (uint32_t)k;
+    } else {
+      return min(off0 + i * copy_stride, b_last);
+    }
   };
   auto copy_tile = [&](int kt, int stage) {
     const int ko = kt * kBK;
@@ -834,7 +856,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
                                        AOPS_LDS_PTR(da + i * kWaves * 512), 16, 0, 0);
 #pragma unroll
     for (int i = 0; i < kBCopies; ++i)
-      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(b_base + ko + min(off0 + i * copy_stride, b_last)),
+      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(b_base + ko + b_offset(i)),
                                        AOPS_LDS_PTR(db + i * kWaves * 512), 16, 0, 0);
   };
 
@@ -954,8 +976,41 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     // (fq = 0, 1) exchange halves: v_permlane32_swap trades the upper 32 lanes of its first
     // operand for the lower 32 lanes of its second, after which lane fq holds the 8 consecutive
     // columns of group g+fq.
-    const int col_w = cur.n_tile * BN + wn * 32 * NB;
     const int m_w = 32 * wm + fm;
+    if constexpr (SWIGLU) {
+      const int col_w = cur.n_tile * BNO + wn * 32;
+#pragma unroll
+      for (int i = 0; i < MB; ++i) {
+        const int m = m_w + 64 * i;
+        if (i < live && col_w < n_out) {  // wave uniform
+          const bool row_ok = m < tile_rows;
+          f16* yrow = y + (int64_t)(cur.row_begin + m) * n_out + col_w + 8 * fq;
+#pragma unroll
+          for (int gp = 0; gp < 2; ++gp) {
+            f16x4 p0, p1;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float g = acc[i][0][8 * gp + e];
+              const float u = acc[i][1][8 * gp + e];
+              const float ex = __builtin_amdgcn_exp2f(-1.4426950408889634f * g);
+              const f16 o = (f16)(g * u * __builtin_amdgcn_rcpf(1.0f + ex));
+              if (e < 4) p0[e] = o; else p1[e - 4] = o;
+            }
+            const u32x2 d0 = __builtin_bit_cast(u32x2, p0);
+            const u32x2 d1 = __builtin_bit_cast(u32x2, p1);
+            const auto lo = __builtin_amdgcn_permlane32_swap(d0[0], d1[0], false, false);
+            const auto hi = __builtin_amdgcn_permlane32_swap(d0[1], d1[1], false, false);
+            u32x4 out;
+            out[0] = lo[0];
+            out[1] = hi[0];
+            out[2] = lo[1];
+            out[3] = hi[1];
+            if (row_ok) st128(yrow + 16 * gp, __builtin_bit_cast(f16x8, out));
+          }
+        }
+      }
+    } else {
+    const int col_w = cur.n_tile * BN + wn * 32 * NB;
 #pragma unroll
     for (int i = 0; i < MB; ++i) {
       const int m = m_w + 64 * i;
@@ -988,6 +1043,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
         }
       }
     }
+    }
     if (!nxt.valid) break;
     cur = nxt;
   }
@@ -995,7 +1051,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
 }
 
-template <int MB, int NB, int WN>
+template <int MB, int NB, int WN, bool SWIGLU>
 static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* group_list, f16* y,
                                  int64_t rows, int k, int num_experts, int n, hipStream_t stream) {
   constexpr int BM = 64 * MB;
@@ -1014,12 +1070,14 @@ static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* grou
     if (e != hipSuccess) return record_launch_status(e);
     cus[dev] = v > 0 ? v : 8;
   }
-  const int64_t n_tiles = (n + BN - 1) / BN;
+  constexpr int BNO = SWIGLU ? BN / 2 : BN;
+  const int64_t n_out = SWIGLU ? n / 2 : n;
+  const int64_t n_tiles = (n_out + BNO - 1) / BNO;
   const int64_t max_work = ((rows + BM - 1) / BM + num_experts) * n_tiles;
   int64_t grid = cus[dev] < max_work ? cus[dev] : max_work;
   grid = grid / kXcds * kXcds;
   if (grid < kXcds) grid = kXcds;
-  auto kernel = grouped_matmul_persistent_kernel<MB, NB, WN>;
+  auto kernel = grouped_matmul_persistent_kernel<MB, NB, WN, SWIGLU>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -1118,7 +1176,7 @@ extern "C" int aops_grouped_matmul_f16(const void* x, const void* w, const int64
   if (variant == 6 && (k % 128 != 0 || k < 256)) variant = 1;  // the persistent kernel's k loop
   switch (variant) {
     case 6:  // 320 x 256 tiles, eight waves, one persistent workgroup per CU
-      return gmm_persistent_launch<5, 2, 4>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts,
+      return gmm_persistent_launch<5, 2, 4, false>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts,
                                             (int)n, s);
     case 1:  // 320 x 256 tiles, eight waves, operands copied HBM -> LDS directly
       return gmm_dma_launch<5, 2, 4>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n,
@@ -1132,4 +1190,21 @@ extern "C" int aops_grouped_matmul_f16(const void* x, const void* w, const int64
     default:  // 64 x 64 tiles
       return gmm_launch<1, 1, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
   }
+}
+
+extern "C" int aops_grouped_matmul_swiglu_f16(const void* x, const void* w, const int64_t* group_list,
+                                              void* y, int64_t rows, int64_t k, int64_t num_experts,
+                                              int64_t n, void* stream) {
+  using namespace aops;
+  if (rows < 0 || k <= 0 || n <= 0 || num_experts < 0 || k % 128 != 0 || k < 256 || n % 64 != 0)
+    return AOPS_ERR_INVALID_ARGUMENT;
+  // 32-bit per-lane offsets: (n/2 + 32) weight rows of k elements must fit
+  if (rows > 0x7fffffff - 4096 || k > (1 << 22) || n > 0x7fffffff || num_experts > (1 << 20) ||
+      (n / 2 + 320) * k > 0x7fffffffLL)
+    return AOPS_ERR_INVALID_ARGUMENT;
+  if (rows == 0 || num_experts == 0) return AOPS_OK;
+  if (!x || !w || !group_list || !y) return AOPS_ERR_INVALID_ARGUMENT;
+  return gmm_persistent_launch<5, 2, 4, true>(
+      static_cast<const f16*>(x), static_cast<const f16*>(w), group_list, static_cast<f16*>(y), rows,
+      (int)k, (int)num_experts, (int)n, static_cast<hipStream_t>(stream));
 }

@@ -318,6 +318,35 @@ def _gmm_entry(L, ops, R, dev, cpu, op, config, x, w_storage, gl, note=None, che
     return e, ys[-1]
 
 
+def _gmm_swiglu_entry(L, ops, dev, config, x, w_storage, gl, h_dev):
+    """Fused gate_up + SwiGLU (extension, no reference counterpart): timed like the other GEMMs and
+    checked against the device's own two-operator chain (which is checked against the oracle)."""
+    import torch
+
+    rows, K = x.shape
+    E, N, _ = w_storage.shape
+    end = int(gl[-1])
+    flops = 2 * end * K * N
+    alg = rows * K * 2 + E * N * K * 2 + end * (N // 2) * 2 + E * 8
+    xd, wd, gd = x.to(dev), w_storage.to(dev), gl.to(dev)
+    n = n_sets_for(alg, lo=1, hi=8)
+    xs = [xd] + [xd.clone() for _ in range(n - 1)]
+    ws = [wd] + [wd.clone() for _ in range(n - 1)]
+    ys = [torch.empty(rows, N // 2, dtype=torch.float16, device=dev) for _ in range(n)]
+
+    def mk(i):
+        return lambda: L.check(L.lib.aops_grouped_matmul_swiglu_f16(xs[i].data_ptr(), ws[i].data_ptr(), gd.data_ptr(),
+                                                                   ys[i].data_ptr(), rows, K, E, N, L.stream()))
+
+    med, mn = time_graph([mk(i) for i in range(n)], min_launches=40)
+    two = ops.swiglu(h_dev)
+    torch.testing.assert_close(ys[-1][:end].float(), two[:end].float(), rtol=2e-2, atol=2e-2)
+    e = entry("grouped_matmul_swiglu", config, f"x [{rows},{K}] @ w [{E},{K},{N}] f16 -> [{rows},{N // 2}]", "mfma", alg,
+              flops, med, mn, None, None, torch.get_num_threads(),
+              "extension: activation fused into the GEMM epilogue, replaces the gate_up and swiglu lines above")
+    return e
+
+
 def bench_moe(L, ops, R, dev, cpu):
     import torch
 
@@ -335,6 +364,7 @@ def bench_moe(L, ops, R, dev, cpu):
     out = []
     e1, h_dev = _gmm_entry(L, ops, R, dev, cpu, "grouped_matmul", "4: MoE gate_up", x, w1, gl)
     out.append(e1)
+    e_fused = _gmm_swiglu_entry(L, ops, dev, "4: MoE gate_up + activation, fused", x, w1, gl, h_dev)
     del w1
     h = ops.swiglu(h_dev)
     # swiglu at the MoE shape
@@ -353,6 +383,7 @@ def bench_moe(L, ops, R, dev, cpu):
     del hs, ys
     e2, _ = _gmm_entry(L, ops, R, dev, cpu, "grouped_matmul", "4: MoE down", h.cpu(), w2, gl)
     out.append(e2)
+    out.append(e_fused)
     tot_flops = e1["algorithmic_flops"] + e2["algorithmic_flops"]
     tot_us = e1["gpu_us"] + e2["gpu_us"]
     out.append({

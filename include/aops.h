@@ -103,6 +103,22 @@ int aops_grouped_matmul_f16(const void* x, const void* w, const int64_t* group_l
                             void* stream);
 
 /*
+ * Grouped matmul of a gate_up projection with the SwiGLU activation fused into its epilogue:
+ *   h = x[rows of expert e] (fp32 accumulate) @ w[e]^T          (never stored)
+ *   y[r, c] = f16( silu(h[r, c]) * h[r, n/2 + c] ),  c < n/2
+ * x, w, group_list as for aops_grouped_matmul_f16; y: [rows, n/2].  Equal, up to the fp16 rounding
+ * of h that it skips, to aops_grouped_matmul_f16 followed by aops_swiglu_f16, without the
+ * [rows, n] intermediate.  k must be a multiple of 128 and at least 256, n a multiple of 64;
+ * other shapes return AOPS_ERR_INVALID_ARGUMENT (call the two operators instead).
+ * Replaces the chain aclnnGroupedMatMulEx -> aclnnSwiGluEx of an expert MLP (reference
+ * csrc/ffi/ops.cpp:211-218 and 138-145, chained as in benchmark/test_mlp.py:37-41); the reference
+ * has no fused operator.
+ */
+int aops_grouped_matmul_swiglu_f16(const void* x, const void* w, const int64_t* group_list, void* y,
+                                   int64_t rows, int64_t k, int64_t num_experts, int64_t n,
+                                   void* stream);
+
+/*
  * Paged-attention decode (one query token per sequence).
  * q, o: [bs, num_heads, head_dim]; key_cache, value_cache:
  * [num_blocks, num_kv_heads*head_dim/16, block_size, 16]; block_tables: int32

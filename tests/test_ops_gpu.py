@@ -256,6 +256,36 @@ def test_grouped_matmul_every_kernel(ops, dev, monkeypatch, variant, rows, K, N,
     assert torch.all(y[end:] == 5.0)
 
 
+@pytest.mark.parametrize(
+    "rows,K,N,E,counts",
+    [
+        (1300, 256, 192, 6, [0, 1, 700, 0, 330, 200]),   # ragged groups, N/2 = 96 (three column blocks of the last tile)
+        (4096, 512, 1536, 64, None),                      # several work items per workgroup
+        (700, 2048, 1536, 1, [650]),                      # one expert, rows past the group untouched
+        (300, 192, 128, 3, [100, 100, 100]),              # K not a multiple of 128: two-kernel path
+    ],
+)
+def test_grouped_matmul_swiglu_fused(ops, dev, rows, K, N, E, counts):
+    """Fused gate_up + SwiGLU against the oracle chain swiglu_ref(grouped_matmul_ref(...)) with the fp32
+    intermediate, and against the unfused device chain."""
+    import ascend910a_extras.fused as fused
+    x, w, gl = _gmm_case(rows, K, N, E, seed=11, counts=counts)
+    end = int(gl[-1])
+    xd, wd, gd = x.to(dev), w.to(dev), gl.to(dev)
+    y = fused.grouped_matmul_swiglu(xd, wd, gd)
+    assert y.shape == (rows, N // 2) and y.dtype == H
+    h = torch.zeros(rows, N)
+    prev = 0
+    for e in range(E):
+        t = int(gl[e])
+        h[prev:t] = x[prev:t].float() @ w[e].float()
+        prev = t
+    ref = (torch.nn.functional.silu(h[:, : N // 2]) * h[:, N // 2:]).half()
+    torch.testing.assert_close(y.cpu()[:end].float(), ref[:end].float(), **GMM_TOL)
+    two = ops.swiglu(ops.grouped_matmul(xd, wd, gd))
+    torch.testing.assert_close(y[:end].float(), two[:end].float(), **GMM_TOL)
+
+
 def test_dense_mlp_chain(ops, dev):
     """benchmark/test_mlp.py:37-41 through grouped_matmul with one expert (reduced width)."""
     g = _gen(0)
