@@ -32,6 +32,10 @@ _SIGNATURES = {
     "aops_swiglu_f16": (ctypes.c_int, [_vp, _vp, _i64, _i64, _vp]),
     "aops_rope_neox_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_reshape_and_cache_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "aops_rope_reshape_and_cache_f16": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
+    ),
     "aops_grouped_matmul_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_grouped_matmul_swiglu_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_paged_attention_workspace": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64]),
@@ -361,6 +365,56 @@ def paged_attention(q, key_cache, value_cache, block_tables, context_lens):
     )
     _status("paged_attention", code)
     return o
+
+
+def rope_reshape_and_cache(q, k, v, position_ids, cos_cache, sin_cache, key_cache, value_cache, slot_indices,
+                           return_k=False):
+    """``out_q, out_k = rope(...); reshape_and_cache(out_k, v, key_cache, value_cache, slot_indices)`` in
+    one kernel (the order of reference csrc/ffi/graph.cpp:255-270).  Returns out_q, or [out_q, out_k]
+    with ``return_k``.  Not part of the reference's surface."""
+    name = "rope_reshape_and_cache"
+    _check(
+        q.dim() == 3 and k.dim() == 3 and v.dim() == 3 and position_ids.dim() == 1 and cos_cache.dim() == 2
+        and sin_cache.dim() == 2 and key_cache.dim() == 4 and value_cache.dim() == 4 and slot_indices.dim() == 1,
+        f"{name}: q, k, v must be 3D, position_ids and slot_indices 1D, cos_cache and sin_cache 2D, caches 4D",
+    )
+    _check(
+        all(t.is_contiguous() for t in (q, k, v, position_ids, cos_cache, sin_cache, key_cache, value_cache, slot_indices)),
+        f"{name}: all input tensors must be contiguous",
+    )
+    bs, num_heads, head_dim = q.shape
+    num_kv_heads = k.size(1)
+    _check(k.size(0) == bs and k.size(2) == head_dim and v.shape == k.shape,
+           f"{name}: k and v must be [bs, num_kv_heads, head_dim] matching q")
+    _check(position_ids.size(0) == bs and slot_indices.size(0) == bs,
+           f"{name}: position_ids and slot_indices must have one entry per token")
+    _check(head_dim % 16 == 0, f"{name}: head_dim must be a multiple of 16, got {head_dim}")
+    _check(cos_cache.size(1) == head_dim // 2 and sin_cache.shape == cos_cache.shape,
+           f"{name}: cos_cache and sin_cache must be [max_position, head_dim/2]")
+    num_blocks, nh16, block_size, chunk = key_cache.shape
+    _check(
+        chunk == 16 and nh16 * 16 == num_kv_heads * head_dim and value_cache.shape == key_cache.shape,
+        f"{name}: caches must be [num_blocks, num_kv_heads*head_dim/16, block_size, 16], got "
+        f"{tuple(key_cache.shape)} and {tuple(value_cache.shape)}",
+    )
+    _require_device(
+        name,
+        {
+            "q": (q, torch.float16), "k": (k, torch.float16), "v": (v, torch.float16),
+            "position_ids": (position_ids, torch.int32), "cos_cache": (cos_cache, torch.float16),
+            "sin_cache": (sin_cache, torch.float16), "key_cache": (key_cache, torch.float16),
+            "value_cache": (value_cache, torch.float16), "slot_indices": (slot_indices, torch.int32),
+        },
+    )
+    out_q = torch.empty_like(q)
+    out_k = torch.empty_like(k) if return_k else None
+    code = _lib.aops_rope_reshape_and_cache_f16(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(position_ids), _ptr(cos_cache), _ptr(sin_cache), _ptr(out_q),
+        _ptr(out_k) if return_k else None, _ptr(key_cache), _ptr(value_cache), _ptr(slot_indices),
+        bs, num_heads, num_kv_heads, head_dim, num_blocks, block_size, _stream(q.device),
+    )
+    _status(name, code)
+    return [out_q, out_k] if return_k else out_q
 
 
 def print_info(device_id: int) -> None:

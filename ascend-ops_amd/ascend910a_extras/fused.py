@@ -12,3 +12,23 @@ def grouped_matmul_swiglu(x: torch.Tensor, w: torch.Tensor, group_list: torch.Te
     the gate_up projection of an expert MLP (reference ``benchmark/test_mlp.py:37-41``) with the
     activation applied to the fp32 accumulators.  Returns ``[rows, N/2]``."""
     return _C.grouped_matmul_swiglu(x, w, group_list)
+
+
+def rope_reshape_and_cache(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    position_ids: torch.Tensor,
+    cos_cache: torch.Tensor,
+    sin_cache: torch.Tensor,
+    key_cache: torch.Tensor,
+    value_cache: torch.Tensor,
+    slot_indices: torch.Tensor,
+    return_k: bool = False,
+):
+    """The decode step's ``out_q, out_k = ops.rope(q, k, position_ids, cos_cache, sin_cache)`` followed by
+    ``ops.reshape_and_cache(out_k, v, key_cache, value_cache, slot_indices)`` (reference
+    ``csrc/ffi/graph.cpp:255-270``) in one launch, bit for bit.  Returns ``out_q`` (``[out_q, out_k]``
+    with ``return_k``); the caches are updated in place."""
+    return _C.rope_reshape_and_cache(q, k, v, position_ids, cos_cache, sin_cache, key_cache, value_cache,
+                                     slot_indices, return_k)

@@ -25,6 +25,7 @@ SOURCES = [
     "add_rms_norm.hip",
     "swiglu.hip",
     "rope.hip",
+    "rope_cache.hip",
     "reshape_and_cache.hip",
     "paged_attention.hip",
     "grouped_matmul.hip",

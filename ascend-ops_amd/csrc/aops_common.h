@@ -58,6 +58,18 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Rotate-half rotation of 8 (x1, x2) pairs in fp32 with one rounding.  The products are combined
+// with explicit fused multiply-adds so that every kernel that rotates produces the same bits.
+__device__ __forceinline__ void rope_rotate8(const f16x8& x1, const f16x8& x2, const f16x8& cs,
+                                             const f16x8& sn, f16x8& o1, f16x8& o2) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float a = (float)x1[j], b = (float)x2[j], c = (float)cs[j], s = (float)sn[j];
+    o1[j] = (f16)__builtin_fmaf(a, c, -(b * s));
+    o2[j] = (f16)__builtin_fmaf(b, c, a * s);
+  }
+}
+
 // Launch-status bookkeeping shared by the host launchers.
 int record_launch_status(hipError_t e);
 

@@ -37,12 +37,7 @@ __global__ __launch_bounds__(256) void rope_neox_kernel(
   const f16x8 cs = ld128(cos_cache + pos * half + c * 8);
   const f16x8 sn = ld128(sin_cache + pos * half + c * 8);
   f16x8 o1, o2;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const float a = (float)x1[j], bb = (float)x2[j], cc = (float)cs[j], ss = (float)sn[j];
-    o1[j] = (f16)(a * cc - bb * ss);
-    o2[j] = (f16)(bb * cc + a * ss);
-  }
+  rope_rotate8(x1, x2, cs, sn, o1, o2);
   st128_stream(dst + c * 8, o1);
   st128_stream(dst + half + c * 8, o2);
 }

@@ -472,6 +472,14 @@ class PagedAttentionWorkload:
         ops.reshape_and_cache(ok, d["v"], self.kcs[i % self.n_sets], self.vcs[i % self.n_sets], d["slots"])
         return ops.paged_attention(oq, self.kcs[i % self.n_sets], self.vcs[i % self.n_sets], d["bt"], d["ctx"])
 
+    def pipeline_fused(self, ops, i=0):
+        import ascend910a_extras.fused as fused
+
+        d = self.d
+        kc, vc = self.kcs[i % self.n_sets], self.vcs[i % self.n_sets]
+        oq = fused.rope_reshape_and_cache(d["q"], d["k"], d["v"], d["pos"], d["cos"], d["sin"], kc, vc, d["slots"])
+        return ops.paged_attention(oq, kc, vc, d["bt"], d["ctx"])
+
 
 def bench_paged_attention(L, ops, R, dev, cpu, wl):
     import torch
@@ -504,6 +512,9 @@ def bench_paged_attention(L, ops, R, dev, cpu, wl):
     # whole decode step: rope -> cache write -> attention (graph of the three C-ABI calls via the API)
     pipe = time_eager([(lambda i=i: wl.pipeline(ops, i)) for i in range(wl.n_sets)], 5, 40)
     e["pipeline_rope_cache_attention_api_eager_us"] = round(pipe, 2)
+    pipe2 = time_eager([(lambda i=i: wl.pipeline_fused(ops, i)) for i in range(wl.n_sets)], 5, 40)
+    e["pipeline_fused_rope_cache_then_attention_api_eager_us"] = round(pipe2, 2)
+    torch.testing.assert_close(wl.pipeline_fused(ops, 0).float(), wl.pipeline(ops, 0).float(), rtol=0, atol=0)
     return e
 
 

@@ -88,6 +88,25 @@ int aops_reshape_and_cache_f16(const void* key, const void* value, void* key_cac
                                void* stream);
 
 /*
+ * Decode-step fusion of the two operators above: out_q = rope(q); the rotated k and the untouched v
+ * of token b go straight to slot slot_indices[b] of the paged caches.  Bit for bit the result of
+ * aops_rope_neox_f16 followed by aops_reshape_and_cache_f16 (rotary dimension == head_dim, one
+ * position and one slot per token).  out_k may be NULL; if not, it also receives the rotated k.
+ * q, out_q: [bs, num_heads, head_dim]; k, v, out_k: [bs, num_kv_heads, head_dim]; caches:
+ * [num_blocks, num_kv_heads*head_dim/16, block_size, 16]; position_ids, slot_indices: int32 [bs].
+ * Replaces the pair aclnnRopeEx -> aclnnReshapeAndCacheEx in the order the reference's decoder
+ * layer runs them (reference csrc/ffi/graph.cpp:255-270; csrc/ffi/ops.cpp:76-83 and 387-396); the
+ * reference has no fused operator.
+ */
+int aops_rope_reshape_and_cache_f16(const void* q, const void* k, const void* v,
+                                    const int32_t* position_ids, const void* cos_cache,
+                                    const void* sin_cache, void* out_q, void* out_k,
+                                    void* key_cache, void* value_cache,
+                                    const int32_t* slot_indices, int64_t bs, int64_t num_heads,
+                                    int64_t num_kv_heads, int64_t head_dim, int64_t num_blocks,
+                                    int64_t block_size, void* stream);
+
+/*
  * Grouped (per-expert) matmul over expert-sorted rows.
  * x: [rows, k]; w: [num_experts, n, k] (each expert's weight stored N-major, K contiguous --
  * the logical [E, K, N] tensor with stride(1)==1, stride(2)==K); group_list: int64

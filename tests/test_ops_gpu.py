@@ -169,6 +169,41 @@ def test_reshape_and_cache_skips_bad_slots_and_roundtrips(ops, dev):
     assert torch.count_nonzero(got) == 0
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,D,NB,P", [(64, 32, 8, 128, 2304, 128), (5, 6, 2, 64, 7, 16), (3, 1, 1, 16, 4, 8), (17, 16, 16, 256, 9, 32)])
+def test_rope_reshape_and_cache_fused_equals_the_chain(ops, dev, B, Hq, Hkv, D, NB, P):
+    """One launch against rope -> reshape_and_cache: q, k and both caches bit for bit, including a slot that is
+    out of range (skipped by both) and cache contents that must stay untouched; and against the oracle."""
+    import ascend910a_extras.fused as fused
+    g = _gen(5)
+    q = torch.randn(B, Hq, D, generator=g).half()
+    k = torch.randn(B, Hkv, D, generator=g).half()
+    v = torch.randn(B, Hkv, D, generator=g).half()
+    cos, sin = R.build_cos_sin_cache(512, D, theta=1e6)
+    pos = torch.randint(0, 512, (B,), generator=g).int()
+    slots = torch.randperm(NB * P, generator=g)[:B].int()
+    slots[B // 2] = NB * P + 3          # skipped
+    kc0 = torch.randn(NB, Hkv * D // 16, P, 16, generator=g).half()
+    vc0 = torch.randn(NB, Hkv * D // 16, P, 16, generator=g).half()
+    qd, kd, vd, posd, cosd, sind, sld = (t.to(dev) for t in (q, k, v, pos, cos, sin, slots))
+    kc_a, vc_a = kc0.to(dev), vc0.to(dev)
+    oq_a, ok_a = ops.rope(qd, kd, posd, cosd, sind)
+    ops.reshape_and_cache(ok_a, vd, kc_a, vc_a, sld)
+    kc_b, vc_b = kc0.to(dev), vc0.to(dev)
+    oq_b, ok_b = fused.rope_reshape_and_cache(qd, kd, vd, posd, cosd, sind, kc_b, vc_b, sld, return_k=True)
+    assert torch.equal(oq_a, oq_b) and torch.equal(ok_a, ok_b)
+    assert torch.equal(kc_a, kc_b) and torch.equal(vc_a, vc_b)
+    kc_c, vc_c = kc0.to(dev), vc0.to(dev)
+    oq_c = fused.rope_reshape_and_cache(qd, kd, vd, posd, cosd, sind, kc_c, vc_c, sld)
+    assert torch.equal(oq_c, oq_a) and torch.equal(kc_c, kc_a) and torch.equal(vc_c, vc_a)
+    # oracle: rotation within tolerance; the cache holds exactly what the device rotation produced
+    rq, rk = R.rope_ref(q, k, pos, cos, sin)
+    torch.testing.assert_close(oq_b.cpu().float(), rq.float(), **TOL)
+    torch.testing.assert_close(ok_b.cpu().float(), rk.float(), **TOL)
+    kc_ref, vc_ref = kc0.clone(), vc0.clone()
+    R.reshape_and_cache_ref(ok_b.cpu(), kc_ref, slots, v, vc_ref)
+    assert torch.equal(kc_b.cpu(), kc_ref) and torch.equal(vc_b.cpu(), vc_ref)
+
+
 # ----------------------------------------------------------------------------- grouped_matmul
 def _gmm_case(rows, K, N, E, seed, counts=None, wstd=0.02):
     g = _gen(seed)
