@@ -83,6 +83,15 @@ def test_c_abi_rejects_bad_sizes_without_touching_the_gpu():
     assert lib.aops_grouped_matmul_f16(None, None, None, None, 16, 100, 2, 64, None) == -1
     assert lib.aops_grouped_matmul_f16(None, None, None, None, 0, 64, 2, 64, None) == 0
     assert lib.aops_paged_attention_f16(None, None, None, None, None, None, None, 0, 2, 8, 2, 72, 128, 4, 16, None) == -1
+    # fused extensions
+    assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 192, 2, 128, None) == -1   # k % 128
+    assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 128, 2, 128, None) == -1   # k < 256
+    assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 256, 2, 128, None) == -1   # null pointers
+    assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 0, 256, 2, 128, None) == 0
+    n = [None] * 11
+    assert lib.aops_rope_reshape_and_cache_f16(*n, 2, 4, 2, 24, 8, 16, None) == -1                   # head_dim % 16
+    assert lib.aops_rope_reshape_and_cache_f16(*n, 2, 4, 2, 64, 8, 16, None) == -1                   # null pointers
+    assert lib.aops_rope_reshape_and_cache_f16(*n, 0, 4, 2, 64, 8, 16, None) == 0
 
 
 H = torch.float16
@@ -127,6 +136,14 @@ def test_argument_checks_follow_the_reference(ops):
     # paged_attention: shapes the reference assumes silently
     _raises(ops.paged_attention, torch.zeros(2, 8, 128, dtype=H), torch.zeros(4, 16, 128, 8, dtype=H),
             torch.zeros(4, 16, 128, 8, dtype=H), torch.zeros(2, 2, dtype=torch.int32), torch.zeros(2, dtype=torch.int32), match="16")
+    # fused extensions share the checks of the operators they chain
+    import ascend910a_extras.fused as fused
+    _raises(fused.grouped_matmul_swiglu, x, torch.zeros(2, 64, 128, dtype=H), gl, match="K-major")
+    bad_cache = torch.zeros(3, 4, 16, 16, dtype=H)
+    _raises(fused.rope_reshape_and_cache, q, k, k, torch.zeros(2, dtype=torch.int32), cs, cs, bad_cache, bad_cache,
+            torch.zeros(2, dtype=torch.int32), match="caches must be")
+    _raises(fused.rope_reshape_and_cache, q, k, k[:1], torch.zeros(2, dtype=torch.int32), cs, cs, cache, cache,
+            torch.zeros(2, dtype=torch.int32), match="k and v must be")
     # valid arguments on the CPU are refused: there is no CPU implementation to fall back to
     _raises(ops.swiglu, torch.zeros(4, 128, dtype=H), match="GPU device")
     _raises(ops.add_rms_norm, torch.zeros(4, 64, dtype=H), torch.zeros(4, 64, dtype=H), torch.zeros(64, dtype=H), 1e-6, match="GPU device")
