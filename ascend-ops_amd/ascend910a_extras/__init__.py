@@ -9,5 +9,6 @@ CPU or eager fallback.
 from . import ascend910a_extras_C  # noqa: F401  (loads libaops.so)
 from . import ops  # noqa: F401
 from . import fused  # noqa: F401
+from . import moe  # noqa: F401
 
-__all__ = ["ops", "fused", "ascend910a_extras_C"]
+__all__ = ["ops", "fused", "moe", "ascend910a_extras_C"]

@@ -38,6 +38,10 @@ _SIGNATURES = {
     ),
     "aops_grouped_matmul_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_grouped_matmul_swiglu_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "aops_moe_sort_workspace": (_sz, [_i64, _i64]),
+    "aops_moe_sort_i32": (ctypes.c_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "aops_moe_gather_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "aops_moe_combine_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_paged_attention_workspace": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64]),
     "aops_paged_attention_f16": (
         ctypes.c_int,
@@ -415,6 +419,60 @@ def rope_reshape_and_cache(q, k, v, position_ids, cos_cache, sin_cache, key_cach
     )
     _status(name, code)
     return [out_q, out_k] if return_k else out_q
+
+
+def moe_sort(topk_ids, num_experts):
+    """Stable sort of the flattened routing by expert: (sorted_idx, inverse_idx, group_list)."""
+    _check(topk_ids.dim() in (1, 2) and topk_ids.is_contiguous(), "moe_sort: topk_ids must be a contiguous 1D or 2D tensor")
+    _check(0 < num_experts <= 4095, f"moe_sort: num_experts must be in 1..4095, got {num_experts}")
+    _require_device("moe_sort", {"topk_ids": (topk_ids, torch.int32)})
+    n = topk_ids.numel()
+    dev = topk_ids.device
+    sorted_idx = torch.empty(n, dtype=torch.int32, device=dev)
+    inverse_idx = torch.empty(n, dtype=torch.int32, device=dev)
+    group_list = torch.empty(num_experts, dtype=torch.int64, device=dev)
+    ws_bytes = _lib.aops_moe_sort_workspace(n, num_experts)
+    _check(ws_bytes > 0, f"moe_sort: unsupported size n={n}, num_experts={num_experts}")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    code = _lib.aops_moe_sort_i32(_ptr(topk_ids), n, num_experts, _ptr(sorted_idx), _ptr(inverse_idx), _ptr(group_list),
+                                  _ptr(ws), ws_bytes, _stream(dev))
+    _status("moe_sort", code)
+    return sorted_idx, inverse_idx, group_list
+
+
+def moe_gather(x, sorted_idx, group_list, topk):
+    """x_sorted[j] = x[sorted_idx[j] // topk] for the routed rows (later rows are left unwritten)."""
+    _check(x.dim() == 2 and x.is_contiguous() and sorted_idx.dim() == 1 and sorted_idx.is_contiguous()
+           and group_list.dim() == 1 and group_list.is_contiguous(), "moe_gather: x must be 2D, sorted_idx and group_list 1D, all contiguous")
+    _check(topk > 0 and sorted_idx.numel() == x.size(0) * topk,
+           f"moe_gather: sorted_idx must have tokens*topk entries, got {sorted_idx.numel()} for {x.size(0)} tokens, topk {topk}")
+    _check(x.size(1) % 8 == 0, f"moe_gather: hidden must be a multiple of 8, got {x.size(1)}")
+    _require_device("moe_gather", {"x": (x, torch.float16), "sorted_idx": (sorted_idx, torch.int32),
+                                   "group_list": (group_list, torch.int64)})
+    n = sorted_idx.numel()
+    out = torch.empty((n, x.size(1)), dtype=x.dtype, device=x.device)
+    code = _lib.aops_moe_gather_f16(_ptr(x), _ptr(sorted_idx), _ptr(group_list), _ptr(out), n, topk, x.size(1),
+                                    group_list.numel(), _stream(x.device))
+    _status("moe_gather", code)
+    return out
+
+
+def moe_combine(y, inverse_idx, topk_weights, topk_ids, num_experts):
+    """out[t] = sum_k topk_weights[t, k] * y[inverse_idx[t*topk + k]] over the valid expert ids."""
+    _check(y.dim() == 2 and y.is_contiguous() and topk_weights.dim() == 2 and topk_weights.is_contiguous()
+           and topk_ids.shape == topk_weights.shape and topk_ids.is_contiguous() and inverse_idx.is_contiguous(),
+           "moe_combine: y must be 2D, topk_weights and topk_ids [tokens, topk], all contiguous")
+    tokens, topk = topk_weights.shape
+    _check(y.size(0) == tokens * topk and inverse_idx.numel() == tokens * topk,
+           f"moe_combine: y and inverse_idx must have tokens*topk rows, got {y.size(0)} and {inverse_idx.numel()}")
+    _check(y.size(1) % 8 == 0, f"moe_combine: hidden must be a multiple of 8, got {y.size(1)}")
+    _require_device("moe_combine", {"y": (y, torch.float16), "inverse_idx": (inverse_idx, torch.int32),
+                                    "topk_weights": (topk_weights, torch.float32), "topk_ids": (topk_ids, torch.int32)})
+    out = torch.empty((tokens, y.size(1)), dtype=y.dtype, device=y.device)
+    code = _lib.aops_moe_combine_f16(_ptr(y), _ptr(inverse_idx), _ptr(topk_weights), _ptr(topk_ids), _ptr(out), tokens, topk,
+                                     y.size(1), num_experts, _stream(y.device))
+    _status("moe_combine", code)
+    return out
 
 
 def print_info(device_id: int) -> None:

@@ -26,6 +26,7 @@ SOURCES = [
     "swiglu.hip",
     "rope.hip",
     "rope_cache.hip",
+    "moe.hip",
     "reshape_and_cache.hip",
     "paged_attention.hip",
     "grouped_matmul.hip",

@@ -347,6 +347,46 @@ def _gmm_swiglu_entry(L, ops, dev, config, x, w_storage, gl, h_dev):
     return e
 
 
+def _moe_glue_entries(L, dev, E, hidden, tokens, topk):
+    """Routing glue of the expert MLP at the configs[3] shape (extension, no reference operator): device-side
+    stable sort -> group_list, row gather, weighted combine.  Checked against the oracle in tests/test_moe_gpu.py."""
+    import torch
+    import ascend910a_extras.moe as moe
+
+    torch.manual_seed(1)
+    n = tokens * topk
+    ids = torch.randint(0, E, (tokens, topk), dtype=torch.int32).to(dev)
+    wts = torch.rand(tokens, topk).to(dev)
+    x = torch.randn(tokens, hidden).half().to(dev)
+    ws_bytes = L.lib.aops_moe_sort_workspace(n, E)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    s_idx = torch.empty(n, dtype=torch.int32, device=dev)
+    inv = torch.empty(n, dtype=torch.int32, device=dev)
+    gl = torch.empty(E, dtype=torch.int64, device=dev)
+    out = []
+    sort_call = lambda: L.check(L.lib.aops_moe_sort_i32(ids.data_ptr(), n, E, s_idx.data_ptr(), inv.data_ptr(),
+                                                        gl.data_ptr(), ws.data_ptr(), ws_bytes, L.stream()))
+    med, mn = time_graph([sort_call], min_launches=100)
+    out.append(entry("moe_sort", "4: routing sort (extension)", f"ids [{tokens},{topk}] int32, {E} experts", "hbm",
+                     n * 4 * 3 + E * 8, 0, med, mn, None, None, 1, "three launches: histogram, scan, stable scatter"))
+    n_sets = n_sets_for(n * hidden * 2 * 2)
+    xs = [torch.empty(n, hidden, dtype=torch.float16, device=dev) for _ in range(n_sets)]
+    med, mn = time_graph([(lambda i=i: L.check(L.lib.aops_moe_gather_f16(x.data_ptr(), s_idx.data_ptr(), gl.data_ptr(),
+                                                                         xs[i].data_ptr(), n, topk, hidden, E, L.stream())))
+                          for i in range(n_sets)])
+    out.append(entry("moe_gather", "4: row gather into expert order (extension)", f"x [{tokens},{hidden}] -> [{n},{hidden}] f16",
+                     "hbm", tokens * hidden * 2 + n * hidden * 2 + n * 4, 0, med, mn, None, None, 1))
+    outs = [torch.empty(tokens, hidden, dtype=torch.float16, device=dev) for _ in range(n_sets)]
+    med, mn = time_graph([(lambda i=i: L.check(L.lib.aops_moe_combine_f16(xs[i].data_ptr(), inv.data_ptr(), wts.data_ptr(),
+                                                                          ids.data_ptr(), outs[i].data_ptr(), tokens, topk,
+                                                                          hidden, E, L.stream())))
+                          for i in range(n_sets)])
+    out.append(entry("moe_combine", "4: weighted combine to token order (extension)",
+                     f"y [{n},{hidden}] -> [{tokens},{hidden}] f16", "hbm",
+                     n * hidden * 2 + tokens * hidden * 2 + n * 12, 0, med, mn, None, None, 1))
+    return out
+
+
 def bench_moe(L, ops, R, dev, cpu):
     import torch
 
@@ -384,6 +424,7 @@ def bench_moe(L, ops, R, dev, cpu):
     e2, _ = _gmm_entry(L, ops, R, dev, cpu, "grouped_matmul", "4: MoE down", h.cpu(), w2, gl)
     out.append(e2)
     out.append(e_fused)
+    out.extend(_moe_glue_entries(L, dev, E, hidden, tokens, topk))
     tot_flops = e1["algorithmic_flops"] + e2["algorithmic_flops"]
     tot_us = e1["gpu_us"] + e2["gpu_us"]
     out.append({

@@ -138,6 +138,39 @@ int aops_grouped_matmul_swiglu_f16(const void* x, const void* w, const int64_t* 
                                    void* stream);
 
 /*
+ * Routing glue of an expert MLP (no counterpart among the reference's operators: its caller does
+ * these steps; the reference itself only shows the host-side construction of group_list,
+ * benchmark/test_grouped_matmul.py:46-50).
+ *
+ * aops_moe_sort_i32: stable counting sort of n expert ids (the flattened [tokens, topk] routing).
+ *   sorted_idx[j]   = index i of the id that lands at sorted position j (token = i / topk)
+ *   inverse_idx[i]  = j (may be NULL)
+ *   group_list[e]   = number of ids <= e, int64, the cumulative form aops_grouped_matmul_f16 reads
+ * Ids outside [0, num_experts) sort behind every valid id, in their original order, and are not
+ * counted in group_list.  num_experts <= 4095, n < 2^31.  aops_moe_sort_workspace() returns the
+ * bytes of workspace needed (0 = unsupported size).
+ *
+ * aops_moe_gather_f16: out[j, :] = x[sorted_idx[j] / topk, :] for j < group_list[num_experts-1]
+ *   (x: [n / topk, hidden], out: [n, hidden], hidden a multiple of 8; later rows are not written).
+ *
+ * aops_moe_combine_f16: out[t, :] = f16( sum_k weights[t, k] * y[inverse_idx[t*topk + k], :] ) over
+ *   the k with a valid expert id, fp32 accumulation in the order of k
+ *   (y: [tokens*topk, hidden]; weights: fp32 [tokens, topk]; expert_ids: int32 [tokens, topk]).
+ */
+size_t aops_moe_sort_workspace(int64_t n, int64_t num_experts);
+
+int aops_moe_sort_i32(const int32_t* expert_ids, int64_t n, int64_t num_experts, int32_t* sorted_idx,
+                      int32_t* inverse_idx, int64_t* group_list, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
+int aops_moe_gather_f16(const void* x, const int32_t* sorted_idx, const int64_t* group_list, void* out,
+                        int64_t n, int64_t topk, int64_t hidden, int64_t num_experts, void* stream);
+
+int aops_moe_combine_f16(const void* y, const int32_t* inverse_idx, const float* weights,
+                         const int32_t* expert_ids, void* out, int64_t tokens, int64_t topk,
+                         int64_t hidden, int64_t num_experts, void* stream);
+
+/*
  * Paged-attention decode (one query token per sequence).
  * q, o: [bs, num_heads, head_dim]; key_cache, value_cache:
  * [num_blocks, num_kv_heads*head_dim/16, block_size, 16]; block_tables: int32

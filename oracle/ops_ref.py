@@ -243,3 +243,40 @@ def paged_attention_ref(q, key_cache, value_cache, block_tables, context_lens):
         o = torch.einsum("ghj,jgd->ghd", p, v)
         out[b] = o.reshape(hq, d).to(q.dtype)
     return out
+
+
+# --------------------------------------------------------------------------- MoE routing glue
+def moe_sort_ref(topk_ids, num_experts):
+    """Stable sort of the flattened routing by expert, the device-side form of what
+    benchmark/test_grouped_matmul.py:46-50 does on the host (sort the expert ids, count,
+    cumulative sum).  Ids outside ``[0, num_experts)`` sort last and are not counted.
+    Returns ``(sorted_idx int32, inverse_idx int32, group_list int64)``."""
+    flat = topk_ids.reshape(-1).long()
+    key = torch.where((flat < 0) | (flat >= num_experts), torch.full_like(flat, num_experts), flat)
+    order = torch.sort(key, stable=True).indices
+    inverse = torch.empty_like(order)
+    inverse[order] = torch.arange(order.numel())
+    counts = torch.bincount(key, minlength=num_experts + 1)[:num_experts]
+    return order.int(), inverse.int(), counts.cumsum(0).to(torch.int64)
+
+
+def moe_mlp_ref(x, topk_ids, topk_weights, w_gate_up, w_down):
+    """Token-by-token fp32 expert MLP: ``sum_k w[t,k] * down_e(silu(gate_e(x_t)) * up_e(x_t))`` with
+    ``e = topk_ids[t,k]`` (benchmark/test_mlp.py:30-41 per expert); ``w_gate_up`` logical
+    ``[E, hidden, 2*inter]``, ``w_down`` logical ``[E, inter, hidden]``.  Invalid ids contribute nothing."""
+    tokens, topk = topk_ids.shape
+    num_experts = w_gate_up.size(0)
+    inter = w_down.size(1)
+    out = torch.zeros(tokens, w_down.size(2), dtype=torch.float32)
+    xf = x.float()
+    for e in range(num_experts):
+        hit = (topk_ids == e)
+        rows = hit.any(dim=1).nonzero().flatten()
+        if rows.numel() == 0:
+            continue
+        h = xf[rows] @ w_gate_up[e].float()
+        a = torch.nn.functional.silu(h[:, :inter]) * h[:, inter:]
+        y = a @ w_down[e].float()
+        wsum = (topk_weights[rows].float() * hit[rows].float()).sum(dim=1, keepdim=True)
+        out[rows] += wsum * y
+    return out

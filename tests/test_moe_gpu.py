@@ -1,0 +1,83 @@
+"""Routing glue of the expert MLP (device-side sort / gather / combine) against the CPU oracle: the sort is
+integer work and must match a stable torch sort exactly; the gather is a copy (bit-exact); the combine and the
+whole routed MLP are compared in fp32 within the grouped-matmul tolerance."""
+import pytest
+import torch
+
+import oracle.ops_ref as R
+
+pytestmark = pytest.mark.gpu
+H = torch.float16
+
+
+@pytest.mark.parametrize(
+    "tokens,topk,E,invalid",
+    [
+        (4096, 8, 128, False),     # configs[3] routing
+        (1000, 2, 8, True),        # n not a multiple of the slice, ids -1 and E mixed in
+        (1, 1, 1, False),
+        (77, 6, 300, True),        # more experts than lanes of a wave
+        (513, 1, 4095, False),     # largest expert count
+        (20000, 4, 3, False),      # long runs of equal ids
+    ],
+)
+def test_moe_sort_matches_a_stable_sort_exactly(dev, tokens, topk, E, invalid):
+    import ascend910a_extras.moe as moe
+    g = torch.Generator().manual_seed(tokens + E)
+    ids = torch.randint(0, E, (tokens, topk), generator=g, dtype=torch.int32)
+    if invalid:
+        bad = torch.rand(tokens, topk, generator=g) < 0.1
+        ids[bad] = -1
+        ids[0, 0] = E
+    s, inv, gl = moe.moe_sort(ids.to(dev), E)
+    rs, rinv, rgl = R.moe_sort_ref(ids, E)
+    assert torch.equal(gl.cpu(), rgl)
+    assert torch.equal(s.cpu(), rs)
+    assert torch.equal(inv.cpu(), rinv)
+    assert s.dtype == torch.int32 and gl.dtype == torch.int64
+
+
+def test_moe_sort_of_nothing(dev):
+    import ascend910a_extras.moe as moe
+    s, inv, gl = moe.moe_sort(torch.zeros(0, 4, dtype=torch.int32, device=dev), 16)
+    assert s.numel() == 0 and torch.equal(gl.cpu(), torch.zeros(16, dtype=torch.int64))
+
+
+def test_moe_gather_and_combine(dev):
+    import ascend910a_extras.moe as moe
+    g = torch.Generator().manual_seed(3)
+    tokens, topk, E, hidden = 300, 4, 16, 256
+    ids = torch.randint(0, E, (tokens, topk), generator=g, dtype=torch.int32)
+    ids[torch.rand(tokens, topk, generator=g) < 0.15] = -1
+    w = torch.rand(tokens, topk, generator=g)
+    x = torch.randn(tokens, hidden, generator=g).half()
+    s, inv, gl = moe.moe_sort(ids.to(dev), E)
+    xs = moe.moe_gather(x.to(dev), s, gl, topk)
+    end = int(gl[-1])
+    assert end == int((ids >= 0).sum())
+    assert torch.equal(xs.cpu()[:end], x[(s.cpu()[:end] // topk).long()])
+    y = torch.randn(tokens * topk, hidden, generator=g).half()
+    out = moe.moe_combine(y.to(dev), inv, w.to(dev), ids.to(dev), E)
+    ref = torch.zeros(tokens, hidden)
+    for t in range(tokens):
+        for k in range(topk):
+            if ids[t, k] >= 0:
+                ref[t] += w[t, k] * y[int(inv[t * topk + k])].float()
+    torch.testing.assert_close(out.cpu().float(), ref, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("tokens,topk,E,hidden,inter", [(512, 4, 16, 256, 128), (4096, 8, 128, 512, 256)])
+def test_moe_mlp_end_to_end(dev, tokens, topk, E, hidden, inter):
+    import ascend910a_extras.moe as moe
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(tokens, hidden, generator=g).half()
+    logits = torch.randn(tokens, E, generator=g)
+    wts, ids = torch.topk(torch.softmax(logits, -1), topk, dim=-1)
+    wts = (wts / wts.sum(-1, keepdim=True)).float()
+    ids = ids.int()
+    w1 = (torch.randn(E, 2 * inter, hidden, generator=g) / hidden ** 0.5).half().transpose(1, 2)
+    w2 = (torch.randn(E, hidden, inter, generator=g) / inter ** 0.5).half().transpose(1, 2)
+    out = moe.moe_mlp(x.to(dev), ids.to(dev), wts.to(dev), w1.to(dev), w2.to(dev))
+    ref = R.moe_mlp_ref(x, ids, wts, w1, w2)
+    assert out.shape == (tokens, hidden) and out.dtype == H
+    torch.testing.assert_close(out.cpu().float(), ref, rtol=2e-2, atol=2e-2)

@@ -307,3 +307,41 @@ def test_paged_attention_one_dominant_key():
     kd[page, off, 0] = q[0, 0] * 8  # score ~ 8*|q|^2/sqrt(D) dominates
     o = R.paged_attention_ref(q, R.nz_pack(kd), R.nz_pack(vd), bt, lens)
     torch.testing.assert_close(o[0, 0].float(), vd[page, off, 0].float(), rtol=1e-2, atol=1e-2)
+
+
+def test_moe_sort_ref_reduces_to_the_reference_group_list_and_is_a_stable_permutation():
+    torch.manual_seed(4)
+    E, n = 16, 1000
+    ids = torch.randint(0, E, (n // 4, 4), dtype=torch.int32)
+    order, inverse, gl = R.moe_sort_ref(ids, E)
+    # group_list: the reference's own construction (sort, count, cumulative sum; test_grouped_matmul.py:46-50)
+    assert torch.equal(gl, R.make_group_list(ids.reshape(-1), E))
+    flat = ids.reshape(-1)
+    sorted_ids = flat[order.long()]
+    assert torch.all(sorted_ids[1:] >= sorted_ids[:-1])                      # sorted
+    assert torch.equal(torch.sort(order.long()).values, torch.arange(n))     # a permutation
+    same = sorted_ids[1:] == sorted_ids[:-1]
+    assert torch.all(order[1:][same] > order[:-1][same])                     # stable
+    assert torch.equal(inverse.long()[order.long()], torch.arange(n))        # inverse
+    # invalid ids go last, in their original order, and are not counted
+    ids2 = flat.clone(); ids2[::7] = -1; ids2[3] = E
+    o2, _, gl2 = R.moe_sort_ref(ids2, E)
+    bad = ((ids2 < 0) | (ids2 >= E)).nonzero().flatten()
+    assert int(gl2[-1]) == n - bad.numel()
+    assert torch.equal(o2[int(gl2[-1]):].long(), bad)
+
+
+def test_moe_mlp_ref_equals_a_dense_per_token_loop():
+    torch.manual_seed(6)
+    T, topk, E, hidden, inter = 10, 2, 4, 64, 64
+    x = torch.randn(T, hidden).half()
+    ids = torch.randint(0, E, (T, topk), dtype=torch.int32)
+    w = torch.rand(T, topk)
+    w1 = (0.1 * torch.randn(E, hidden, 2 * inter)).half()
+    w2 = (0.1 * torch.randn(E, inter, hidden)).half()
+    ref = torch.zeros(T, hidden)
+    for t in range(T):
+        for k in range(topk):
+            e = int(ids[t, k])
+            ref[t] += w[t, k] * R.mlp_ref(x[t:t + 1], w1[e].t().contiguous(), w2[e].t().contiguous()).float()[0]
+    torch.testing.assert_close(R.moe_mlp_ref(x, ids, w, w1, w2), ref, rtol=2e-2, atol=2e-2)
