@@ -37,6 +37,7 @@ _SIGNATURES = {
         [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
     ),
     "aops_grouped_matmul_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "aops_matmul_nt_f16": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "aops_grouped_matmul_swiglu_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_moe_sort_workspace": (_sz, [_i64, _i64]),
     "aops_moe_sort_i32": (ctypes.c_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
@@ -211,6 +212,24 @@ def grouped_matmul(x, w, group_list):
         _ptr(x), _ptr(w), _ptr(group_list), _ptr(y), num_tokens, dim, num_experts, inner_dim, _stream(x.device)
     )
     _status("grouped_matmul", code)
+    return y
+
+
+def matmul(x, w):
+    """y = x @ w.T for x [m, k], w [n, k]: reference legacy tree _csrc/ffi.cpp:408-442."""
+    _check(x.dim() == 2 and w.dim() == 2, "matmul: input tensors must be 2D")
+    _check(
+        x.size(1) == w.size(1),
+        f"matmul: last dimension of x must match last dimension of w, got {x.size(1)} and {w.size(1)}",
+    )
+    _check(x.is_contiguous() and w.is_contiguous(), "matmul: x and w must be contiguous tensors")
+    m, k = x.shape
+    n = w.size(0)
+    _check(k % 64 == 0 and n % 64 == 0, f"matmul: k and n must be multiples of 64, got k={k} and n={n}")
+    _require_device("matmul", {"x": (x, torch.float16), "w": (w, torch.float16)})
+    y = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    code = _lib.aops_matmul_nt_f16(_ptr(x), _ptr(w), _ptr(y), m, k, n, _stream(x.device))
+    _status("matmul", code)
     return y
 
 

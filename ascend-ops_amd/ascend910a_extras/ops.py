@@ -28,6 +28,12 @@ def grouped_matmul(
     return _C.ops.grouped_matmul(x, w, group_list)
 
 
+def matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """``x @ w.T`` for ``x [m, k]``, ``w [n, k]`` (fp16, fp32 accumulate): the operator of the reference's
+    legacy tree (``_csrc/ffi.cpp:408-442``, ``benchmark/test_matmul.py``), kept under its name."""
+    return _C.matmul(x, w)
+
+
 def add_rms_norm(
     x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, epsilon: float = 1e-5
 ) -> tuple[torch.Tensor, torch.Tensor]:

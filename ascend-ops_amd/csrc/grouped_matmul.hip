@@ -25,6 +25,13 @@ namespace aops {
 constexpr int kBK = 64;   // k extent of one LDS stage
 constexpr int kXcds = 8;
 
+// Cumulative row end of expert e.  group_list == nullptr stands for a single group that holds
+// every row (the dense NT matmul entry point).
+__device__ __forceinline__ int64_t gmm_group_end(const int64_t* __restrict__ group_list, int e,
+                                                 int64_t rows) {
+  return group_list ? group_list[e] : rows;
+}
+
 struct GmmWork {
   int expert;
   int row_begin;  // first row of this m-tile
@@ -44,11 +51,11 @@ __device__ __forceinline__ GmmWork gmm_find_work(const int64_t* __restrict__ gro
   auto clampr = [&](int64_t v) -> int { return (int)(v < 0 ? 0 : (v > rows ? rows : v)); };
   int tiles = 0;
   {
-    int prev = (e0 == 0 || e0 > num_experts) ? 0 : clampr(group_list[e0 - 1]);
+    int prev = (e0 == 0 || e0 > num_experts) ? 0 : clampr(gmm_group_end(group_list, e0 - 1, rows));
     for (int j = 0; j < per; ++j) {
       const int e = e0 + j;
       if (e < num_experts) {
-        const int end = clampr(group_list[e]);
+        const int end = clampr(gmm_group_end(group_list, e, rows));
         if (end > prev) tiles += (end - prev + kBM - 1) / kBM;
         prev = end;
       }
@@ -81,11 +88,11 @@ __device__ __forceinline__ GmmWork gmm_find_work(const int64_t* __restrict__ gro
   const bool mine = work >= lo && work < hi;
   if (mine) {
     int64_t base = lo;
-    int prev = (e0 == 0) ? 0 : clampr(group_list[e0 - 1]);
+    int prev = (e0 == 0) ? 0 : clampr(gmm_group_end(group_list, e0 - 1, rows));
     for (int j = 0; j < per; ++j) {
       const int e = e0 + j;
       if (e >= num_experts) break;
-      const int end = clampr(group_list[e]);
+      const int end = clampr(gmm_group_end(group_list, e, rows));
       const int t = end > prev ? (end - prev + kBM - 1) / kBM : 0;
       const int64_t span = (int64_t)t * n_tiles;
       if (work < base + span) {
@@ -626,7 +633,7 @@ __device__ __forceinline__ GmmPlan gmm_make_plan(const int64_t* __restrict__ gro
   GmmPlan p;
   p.per = (num_experts + kWave - 1) / kWave;
   const int e0 = lane * p.per;
-  int prev = (e0 == 0 || e0 > num_experts) ? 0 : clampr(group_list[e0 - 1]);
+  int prev = (e0 == 0 || e0 > num_experts) ? 0 : clampr(gmm_group_end(group_list, e0 - 1, rows));
   p.bnd[0] = prev;
   p.tiles = 0;
   if (p.per <= kBndCache) {
@@ -635,7 +642,7 @@ __device__ __forceinline__ GmmPlan gmm_make_plan(const int64_t* __restrict__ gro
       const int e = e0 + j;
       int end = prev;  // slots past the lane's experts: empty
       if (j < p.per && e < num_experts) {
-        end = clampr(group_list[e]);
+        end = clampr(gmm_group_end(group_list, e, rows));
         if (end > prev) p.tiles += (end - prev + kBM - 1) / kBM;
       }
       p.bnd[j + 1] = end;
@@ -647,7 +654,7 @@ __device__ __forceinline__ GmmPlan gmm_make_plan(const int64_t* __restrict__ gro
     for (int j = 0; j < p.per; ++j) {
       const int e = e0 + j;
       if (e < num_experts) {
-        const int end = clampr(group_list[e]);
+        const int end = clampr(gmm_group_end(group_list, e, rows));
         if (end > prev) p.tiles += (end - prev + kBM - 1) / kBM;
         prev = end;
       }
@@ -701,11 +708,11 @@ __device__ __forceinline__ GmmWork gmm_locate(const GmmPlan& p,
         prev = end;
       }
     } else {
-      int prev = (e0 == 0) ? 0 : clampr(group_list[e0 - 1]);
+      int prev = (e0 == 0) ? 0 : clampr(gmm_group_end(group_list, e0 - 1, rows));
       for (int j = 0; j < p.per; ++j) {
         const int e = e0 + j;
         if (e >= num_experts) break;
-        const int end = clampr(group_list[e]);
+        const int end = clampr(gmm_group_end(group_list, e, rows));
         const int t = end > prev ? (end - prev + kBM - 1) / kBM : 0;
         const int64_t span = (int64_t)t * n_tiles;
         if (work < base + span) {
@@ -1145,9 +1152,9 @@ static int gmm_launch(const f16* x, const f16* w, const int64_t* group_list, f16
 
 }  // namespace aops
 
-extern "C" int aops_grouped_matmul_f16(const void* x, const void* w, const int64_t* group_list,
-                                       void* y, int64_t rows, int64_t k, int64_t num_experts,
-                                       int64_t n, void* stream) {
+static int aops_grouped_matmul_impl(const void* x, const void* w, const int64_t* group_list, void* y,
+                                    int64_t rows, int64_t k, int64_t num_experts, int64_t n,
+                                    void* stream) {
   using namespace aops;
   if (rows < 0 || k <= 0 || n <= 0 || num_experts < 0 || k % 64 != 0 || n % 64 != 0)
     return AOPS_ERR_INVALID_ARGUMENT;
@@ -1155,7 +1162,7 @@ extern "C" int aops_grouped_matmul_f16(const void* x, const void* w, const int64
   if (rows > 0x7fffffff - 4096 || k > (1 << 22) || n > 0x7fffffff || num_experts > (1 << 20))
     return AOPS_ERR_INVALID_ARGUMENT;
   if (rows == 0 || num_experts == 0) return AOPS_OK;
-  if (!x || !w || !group_list || !y) return AOPS_ERR_INVALID_ARGUMENT;
+  if (!x || !w || !y || (!group_list && num_experts != 1)) return AOPS_ERR_INVALID_ARGUMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const f16* xp = static_cast<const f16*>(x);
   const f16* wp = static_cast<const f16*>(w);
@@ -1192,6 +1199,13 @@ extern "C" int aops_grouped_matmul_f16(const void* x, const void* w, const int64
   }
 }
 
+extern "C" int aops_grouped_matmul_f16(const void* x, const void* w, const int64_t* group_list,
+                                       void* y, int64_t rows, int64_t k, int64_t num_experts,
+                                       int64_t n, void* stream) {
+  if (rows > 0 && num_experts > 0 && !group_list) return AOPS_ERR_INVALID_ARGUMENT;
+  return aops_grouped_matmul_impl(x, w, group_list, y, rows, k, num_experts, n, stream);
+}
+
 extern "C" int aops_grouped_matmul_swiglu_f16(const void* x, const void* w, const int64_t* group_list,
                                               void* y, int64_t rows, int64_t k, int64_t num_experts,
                                               int64_t n, void* stream) {
@@ -1207,4 +1221,12 @@ extern "C" int aops_grouped_matmul_swiglu_f16(const void* x, const void* w, cons
   return gmm_persistent_launch<5, 2, 4, true>(
       static_cast<const f16*>(x), static_cast<const f16*>(w), group_list, static_cast<f16*>(y), rows,
       (int)k, (int)num_experts, (int)n, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int aops_matmul_nt_f16(const void* x, const void* w, void* y, int64_t m, int64_t k, int64_t n,
+                                  void* stream) {
+  if (m < 0 || k <= 0 || n <= 0 || k % 64 != 0 || n % 64 != 0) return AOPS_ERR_INVALID_ARGUMENT;
+  if (m == 0) return AOPS_OK;
+  if (!x || !w || !y) return AOPS_ERR_INVALID_ARGUMENT;
+  return aops_grouped_matmul_impl(x, w, nullptr, y, m, k, 1, n, stream);
 }

@@ -122,6 +122,16 @@ int aops_grouped_matmul_f16(const void* x, const void* w, const int64_t* group_l
                             void* stream);
 
 /*
+ * Dense NT matmul: y = f16( x (fp32 accumulate) @ w^T ), x: [m, k], w: [n, k], y: [m, n]; the
+ * grouped matmul with one group that holds every row (no group_list needed).  k and n must be
+ * multiples of 64.
+ * Replaces matmul of the reference's legacy tree (reference _csrc/ffi.cpp:408-442,
+ * benchmark/test_matmul.py).
+ */
+int aops_matmul_nt_f16(const void* x, const void* w, void* y, int64_t m, int64_t k, int64_t n,
+                       void* stream);
+
+/*
  * Grouped matmul of a gate_up projection with the SwiGLU activation fused into its epilogue:
  *   h = x[rows of expert e] (fp32 accumulate) @ w[e]^T          (never stored)
  *   y[r, c] = f16( silu(h[r, c]) * h[r, n/2 + c] ),  c < n/2

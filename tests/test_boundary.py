@@ -83,6 +83,10 @@ def test_c_abi_rejects_bad_sizes_without_touching_the_gpu():
     assert lib.aops_grouped_matmul_f16(None, None, None, None, 16, 100, 2, 64, None) == -1
     assert lib.aops_grouped_matmul_f16(None, None, None, None, 0, 64, 2, 64, None) == 0
     assert lib.aops_paged_attention_f16(None, None, None, None, None, None, None, 0, 2, 8, 2, 72, 128, 4, 16, None) == -1
+    assert lib.aops_matmul_nt_f16(None, None, None, 16, 100, 64, None) == -1
+    assert lib.aops_matmul_nt_f16(None, None, None, 16, 64, 64, None) == -1    # null pointers
+    assert lib.aops_matmul_nt_f16(None, None, None, 0, 64, 64, None) == 0
+    assert lib.aops_grouped_matmul_f16(ctypes.c_void_p(8), ctypes.c_void_p(8), None, ctypes.c_void_p(8), 4, 64, 1, 64, None) == -1
     # fused extensions
     assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 192, 2, 128, None) == -1   # k % 128
     assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 128, 2, 128, None) == -1   # k < 256

@@ -321,6 +321,17 @@ def test_grouped_matmul_swiglu_fused(ops, dev, rows, K, N, E, counts):
     torch.testing.assert_close(y[:end].float(), two[:end].float(), **GMM_TOL)
 
 
+@pytest.mark.parametrize("m,k,n", [(128, 128, 128), (257, 256, 256), (1, 64, 64), (256, 4096, 1024), (3000, 512, 2048)])
+def test_matmul_nt(ops, dev, m, k, n):
+    """Legacy dense operator (benchmark/test_matmul.py: x [m,k] @ w[n,k]^T), the grouped matmul without a group_list."""
+    g = _gen(m + n)
+    x = torch.randn(m, k, generator=g).half()
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).half()
+    y = ops.matmul(x.to(dev), w.to(dev))
+    assert y.shape == (m, n) and y.dtype == H
+    torch.testing.assert_close(y.cpu().float(), x.float() @ w.float().T, **GMM_TOL)
+
+
 def test_dense_mlp_chain(ops, dev):
     """benchmark/test_mlp.py:37-41 through grouped_matmul with one expert (reduced width)."""
     g = _gen(0)
