@@ -36,6 +36,11 @@ _SIGNATURES = {
         ctypes.c_int,
         [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
     ),
+    "aops_qknorm_rope_reshape_and_cache_f16": (
+        ctypes.c_int,
+        [_vp, _vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+         _i64, _i64, _i64, _i64, _i64, _i64, _vp],
+    ),
     "aops_grouped_matmul_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_matmul_nt_f16": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "aops_grouped_matmul_swiglu_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
@@ -391,11 +396,13 @@ def paged_attention(q, key_cache, value_cache, block_tables, context_lens):
 
 
 def rope_reshape_and_cache(q, k, v, position_ids, cos_cache, sin_cache, key_cache, value_cache, slot_indices,
-                           return_k=False):
+                           return_k=False, q_norm_weight=None, k_norm_weight=None, epsilon=1e-6):
     """``out_q, out_k = rope(...); reshape_and_cache(out_k, v, key_cache, value_cache, slot_indices)`` in
     one kernel (the order of reference csrc/ffi/graph.cpp:255-270).  Returns out_q, or [out_q, out_k]
-    with ``return_k``.  Not part of the reference's surface."""
+    with ``return_k``.  With ``q_norm_weight``/``k_norm_weight`` the per-head RMSNorm of reference
+    csrc/ffi/graph.cpp:252-253 runs in front of the rotation.  Not part of the reference's surface."""
     name = "rope_reshape_and_cache"
+    norm = q_norm_weight is not None or k_norm_weight is not None
     _check(
         q.dim() == 3 and k.dim() == 3 and v.dim() == 3 and position_ids.dim() == 1 and cos_cache.dim() == 2
         and sin_cache.dim() == 2 and key_cache.dim() == 4 and value_cache.dim() == 4 and slot_indices.dim() == 1,
@@ -431,6 +438,21 @@ def rope_reshape_and_cache(q, k, v, position_ids, cos_cache, sin_cache, key_cach
     )
     out_q = torch.empty_like(q)
     out_k = torch.empty_like(k) if return_k else None
+    if norm:
+        _check(q_norm_weight is not None and k_norm_weight is not None, f"{name}: give both norm weights or none")
+        _check(q_norm_weight.shape == (head_dim,) and k_norm_weight.shape == (head_dim,)
+               and q_norm_weight.is_contiguous() and k_norm_weight.is_contiguous(),
+               f"{name}: norm weights must be contiguous [head_dim] tensors")
+        _check(head_dim in (16, 32, 64, 128, 256), f"{name}: the fused norm needs head_dim 16, 32, 64, 128 or 256, got {head_dim}")
+        _require_device(name, {"q_norm_weight": (q_norm_weight, torch.float16), "k_norm_weight": (k_norm_weight, torch.float16)})
+        code = _lib.aops_qknorm_rope_reshape_and_cache_f16(
+            _ptr(q), _ptr(k), _ptr(v), _ptr(q_norm_weight), _ptr(k_norm_weight), float(epsilon), _ptr(position_ids),
+            _ptr(cos_cache), _ptr(sin_cache), _ptr(out_q), _ptr(out_k) if return_k else None, _ptr(key_cache),
+            _ptr(value_cache), _ptr(slot_indices), bs, num_heads, num_kv_heads, head_dim, num_blocks, block_size,
+            _stream(q.device),
+        )
+        _status(name, code)
+        return [out_q, out_k] if return_k else out_q
     code = _lib.aops_rope_reshape_and_cache_f16(
         _ptr(q), _ptr(k), _ptr(v), _ptr(position_ids), _ptr(cos_cache), _ptr(sin_cache), _ptr(out_q),
         _ptr(out_k) if return_k else None, _ptr(key_cache), _ptr(value_cache), _ptr(slot_indices),

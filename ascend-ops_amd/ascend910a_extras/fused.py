@@ -25,10 +25,14 @@ def rope_reshape_and_cache(
     value_cache: torch.Tensor,
     slot_indices: torch.Tensor,
     return_k: bool = False,
+    q_norm_weight: torch.Tensor | None = None,
+    k_norm_weight: torch.Tensor | None = None,
+    epsilon: float = 1e-6,
 ):
     """The decode step's ``out_q, out_k = ops.rope(q, k, position_ids, cos_cache, sin_cache)`` followed by
     ``ops.reshape_and_cache(out_k, v, key_cache, value_cache, slot_indices)`` (reference
     ``csrc/ffi/graph.cpp:255-270``) in one launch, bit for bit.  Returns ``out_q`` (``[out_q, out_k]``
-    with ``return_k``); the caches are updated in place."""
+    with ``return_k``); the caches are updated in place.  With ``q_norm_weight`` and ``k_norm_weight``
+    (``[head_dim]``) the per-head RMSNorm of q and k (``graph.cpp:252-253``) runs first, in the same launch."""
     return _C.rope_reshape_and_cache(q, k, v, position_ids, cos_cache, sin_cache, key_cache, value_cache,
-                                     slot_indices, return_k)
+                                     slot_indices, return_k, q_norm_weight, k_norm_weight, epsilon)

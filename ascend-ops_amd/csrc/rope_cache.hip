@@ -8,12 +8,19 @@
 // Thread map per token: (Hq+Hkv)*D/16 rotation threads (8 pairs each, as in rope_neox_kernel)
 // followed by Hkv*D/8 threads that copy 16 bytes of v.  A rotation thread of a k head writes its two
 // 16-byte results into the cache; threads c and c^1 complete one 32-byte granule.
+//
+// NORM = true puts the per-head RMSNorm of q and k (reference csrc/ffi/graph.cpp:252-253: RMSNorm
+// without residual over head_dim, one weight vector for q and one for k) in front of the rotation:
+// the head_dim/16 threads of a head add up their squares with lane exchanges, the normalised
+// values are rounded to fp16 as the separate operator's output would be, then rotated.
 #include "aops_common.h"
 
 namespace aops {
 
+template <bool NORM>
 __global__ __launch_bounds__(256) void rope_cache_kernel(
     const f16* __restrict__ q, const f16* __restrict__ k, const f16* __restrict__ v,
+    const f16* __restrict__ q_norm_weight, const f16* __restrict__ k_norm_weight, float eps,
     const int32_t* __restrict__ position_ids, const f16* __restrict__ cos_cache,
     const f16* __restrict__ sin_cache, f16* __restrict__ out_q, f16* __restrict__ out_k,
     f16* __restrict__ key_cache, f16* __restrict__ value_cache,
@@ -47,15 +54,34 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(
   const f16x8 cs = ld128(cos_cache + pos * half + c * 8);
   const f16x8 sn = ld128(sin_cache + pos * half + c * 8);
   f16x8 o1, o2;
-  if (head < num_heads) {
-    const int64_t base = ((int64_t)b * num_heads + head) * head_dim;
-    rope_rotate8(ld128_stream(q + base + c * 8), ld128_stream(q + base + half + c * 8), cs, sn, o1, o2);
+  const bool is_q = head < num_heads;
+  const uint32_t hk = head - num_heads;
+  const int64_t base = is_q ? ((int64_t)b * num_heads + head) * head_dim
+                            : ((int64_t)b * num_kv_heads + hk) * head_dim;
+  const f16* src = is_q ? q : k;
+  f16x8 x1 = ld128_stream(src + base + c * 8);
+  f16x8 x2 = ld128_stream(src + base + half + c * 8);
+  if constexpr (NORM) {
+    const f16* nw = is_q ? q_norm_weight : k_norm_weight;
+    const f16x8 w1 = ld128(nw + c * 8);
+    const f16x8 w2 = ld128(nw + half + c * 8);
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ss += (float)x1[j] * (float)x1[j] + (float)x2[j] * (float)x2[j];
+    // the vec_per_head (a power of two) threads of this head are consecutive, aligned lanes
+    for (uint32_t m = 1; m < vec_per_head; m <<= 1) ss += __shfl_xor(ss, (int)m);
+    const float inv_rms = 1.0f / __builtin_sqrtf(ss / (float)head_dim + eps);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      x1[j] = (f16)((float)x1[j] * inv_rms * (float)w1[j]);
+      x2[j] = (f16)((float)x2[j] * inv_rms * (float)w2[j]);
+    }
+  }
+  rope_rotate8(x1, x2, cs, sn, o1, o2);
+  if (is_q) {
     st128_stream(out_q + base + c * 8, o1);
     st128_stream(out_q + base + half + c * 8, o2);
   } else {
-    const uint32_t hk = head - num_heads;
-    const int64_t base = ((int64_t)b * num_kv_heads + hk) * head_dim;
-    rope_rotate8(ld128_stream(k + base + c * 8), ld128_stream(k + base + half + c * 8), cs, sn, o1, o2);
     if (out_k) {
       st128_stream(out_k + base + c * 8, o1);
       st128_stream(out_k + base + half + c * 8, o2);
@@ -70,14 +96,20 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(
 
 }  // namespace aops
 
-extern "C" int aops_rope_reshape_and_cache_f16(
-    const void* q, const void* k, const void* v, const int32_t* position_ids, const void* cos_cache,
-    const void* sin_cache, void* out_q, void* out_k, void* key_cache, void* value_cache,
-    const int32_t* slot_indices, int64_t bs, int64_t num_heads, int64_t num_kv_heads,
-    int64_t head_dim, int64_t num_blocks, int64_t block_size, void* stream) {
-  using namespace aops;
+namespace aops {
+
+static int rope_cache_launch(bool norm, const void* q, const void* k, const void* v,
+                             const void* q_norm_weight, const void* k_norm_weight, float eps,
+                             const int32_t* position_ids, const void* cos_cache, const void* sin_cache,
+                             void* out_q, void* out_k, void* key_cache, void* value_cache,
+                             const int32_t* slot_indices, int64_t bs, int64_t num_heads,
+                             int64_t num_kv_heads, int64_t head_dim, int64_t num_blocks,
+                             int64_t block_size, void* stream) {
   if (bs < 0 || num_heads < 0 || num_kv_heads <= 0 || head_dim <= 0 || head_dim % 16 != 0 ||
       num_blocks < 0 || block_size <= 0 || block_size > 0x7fffffff)
+    return AOPS_ERR_INVALID_ARGUMENT;
+  // the norm's lane exchange needs head_dim/16 threads per head to be a power of two up to 16
+  if (norm && (head_dim > 256 || ((head_dim / 16) & (head_dim / 16 - 1)) != 0))
     return AOPS_ERR_INVALID_ARGUMENT;
   const int64_t num_slots = num_blocks * block_size;
   if (num_slots > 0x7fffffff) return AOPS_ERR_INVALID_ARGUMENT;  // slots are int32
@@ -90,13 +122,40 @@ extern "C" int aops_rope_reshape_and_cache_f16(
       !slot_indices)
     return AOPS_ERR_INVALID_ARGUMENT;
   if (num_heads > 0 && (!q || !out_q)) return AOPS_ERR_INVALID_ARGUMENT;
+  if (norm && (!k_norm_weight || (num_heads > 0 && !q_norm_weight))) return AOPS_ERR_INVALID_ARGUMENT;
   const unsigned grid = (unsigned)((total + 255) / 256);
-  rope_cache_kernel<<<grid, 256, 0, static_cast<hipStream_t>(stream)>>>(
+  auto kernel = norm ? rope_cache_kernel<true> : rope_cache_kernel<false>;
+  kernel<<<grid, 256, 0, static_cast<hipStream_t>(stream)>>>(
       static_cast<const f16*>(q), static_cast<const f16*>(k), static_cast<const f16*>(v),
+      static_cast<const f16*>(q_norm_weight), static_cast<const f16*>(k_norm_weight), eps,
       position_ids, static_cast<const f16*>(cos_cache), static_cast<const f16*>(sin_cache),
       static_cast<f16*>(out_q), static_cast<f16*>(out_k), static_cast<f16*>(key_cache),
       static_cast<f16*>(value_cache), slot_indices, (uint32_t)total, (uint32_t)per_token,
       (uint32_t)rope_threads, (uint32_t)num_heads, (uint32_t)num_kv_heads, (uint32_t)head_dim,
       (uint32_t)block_size, num_slots);
   return record_launch_status(hipGetLastError());
+}
+
+}  // namespace aops
+
+extern "C" int aops_rope_reshape_and_cache_f16(
+    const void* q, const void* k, const void* v, const int32_t* position_ids, const void* cos_cache,
+    const void* sin_cache, void* out_q, void* out_k, void* key_cache, void* value_cache,
+    const int32_t* slot_indices, int64_t bs, int64_t num_heads, int64_t num_kv_heads,
+    int64_t head_dim, int64_t num_blocks, int64_t block_size, void* stream) {
+  return aops::rope_cache_launch(false, q, k, v, nullptr, nullptr, 0.f, position_ids, cos_cache,
+                                 sin_cache, out_q, out_k, key_cache, value_cache, slot_indices, bs,
+                                 num_heads, num_kv_heads, head_dim, num_blocks, block_size, stream);
+}
+
+extern "C" int aops_qknorm_rope_reshape_and_cache_f16(
+    const void* q, const void* k, const void* v, const void* q_norm_weight,
+    const void* k_norm_weight, float epsilon, const int32_t* position_ids, const void* cos_cache,
+    const void* sin_cache, void* out_q, void* out_k, void* key_cache, void* value_cache,
+    const int32_t* slot_indices, int64_t bs, int64_t num_heads, int64_t num_kv_heads,
+    int64_t head_dim, int64_t num_blocks, int64_t block_size, void* stream) {
+  return aops::rope_cache_launch(true, q, k, v, q_norm_weight, k_norm_weight, epsilon, position_ids,
+                                 cos_cache, sin_cache, out_q, out_k, key_cache, value_cache,
+                                 slot_indices, bs, num_heads, num_kv_heads, head_dim, num_blocks,
+                                 block_size, stream);
 }

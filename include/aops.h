@@ -107,6 +107,21 @@ int aops_rope_reshape_and_cache_f16(const void* q, const void* k, const void* v,
                                     int64_t block_size, void* stream);
 
 /*
+ * The same with the per-head RMSNorm of q and k in front of the rotation (reference
+ * csrc/ffi/graph.cpp:252-253: RMSNorm over head_dim without residual, weights [head_dim]):
+ *   qn = f16( q * rsqrt(mean(q^2 over the head) + epsilon) * q_norm_weight ), likewise kn;
+ *   out_q = rope(qn); rotated kn and v go to the caches.
+ * head_dim must be 16, 32, 64, 128 or 256.  Equal to the chain of the separate operators up to the
+ * summation order of the mean (within the operators' tolerance, not bit for bit).
+ */
+int aops_qknorm_rope_reshape_and_cache_f16(
+    const void* q, const void* k, const void* v, const void* q_norm_weight,
+    const void* k_norm_weight, float epsilon, const int32_t* position_ids, const void* cos_cache,
+    const void* sin_cache, void* out_q, void* out_k, void* key_cache, void* value_cache,
+    const int32_t* slot_indices, int64_t bs, int64_t num_heads, int64_t num_kv_heads,
+    int64_t head_dim, int64_t num_blocks, int64_t block_size, void* stream);
+
+/*
  * Grouped (per-expert) matmul over expert-sorted rows.
  * x: [rows, k]; w: [num_experts, n, k] (each expert's weight stored N-major, K contiguous --
  * the logical [E, K, N] tensor with stride(1)==1, stride(2)==K); group_list: int64

@@ -96,6 +96,10 @@ def test_c_abi_rejects_bad_sizes_without_touching_the_gpu():
     assert lib.aops_rope_reshape_and_cache_f16(*n, 2, 4, 2, 24, 8, 16, None) == -1                   # head_dim % 16
     assert lib.aops_rope_reshape_and_cache_f16(*n, 2, 4, 2, 64, 8, 16, None) == -1                   # null pointers
     assert lib.aops_rope_reshape_and_cache_f16(*n, 0, 4, 2, 64, 8, 16, None) == 0
+    m = [None] * 5 + [1e-6] + [None] * 8
+    assert lib.aops_qknorm_rope_reshape_and_cache_f16(*m, 2, 4, 2, 48, 8, 16, None) == -1            # 3 threads per head
+    assert lib.aops_qknorm_rope_reshape_and_cache_f16(*m, 2, 4, 2, 64, 8, 16, None) == -1            # null pointers
+    assert lib.aops_qknorm_rope_reshape_and_cache_f16(*m, 0, 4, 2, 64, 8, 16, None) == 0
 
 
 H = torch.float16

@@ -58,14 +58,16 @@ def test_decoder_layer_decode_step(ops, dev, fused, Hq, Hkv, D):
     hs, res = ops.add_rms_norm(d(x), d(res_in), d(w_ln1), eps)
     qkv = _linear_dev(ops, hs, d(w_qkv), gl)
     q, k, v = qkv.split([q_size, kv_size, kv_size], dim=-1)
-    zq = torch.zeros(B * Hq, D, dtype=H, device=dev)
-    zk = torch.zeros(B * Hkv, D, dtype=H, device=dev)
-    qn = ops.add_rms_norm(q.reshape(B * Hq, D).contiguous(), zq, d(w_qn), eps)[0].view(B, Hq, D)
-    kn = ops.add_rms_norm(k.reshape(B * Hkv, D).contiguous(), zk, d(w_kn), eps)[0].view(B, Hkv, D)
     v3 = v.reshape(B, Hkv, D).contiguous()
-    if fused:
-        oq = F.rope_reshape_and_cache(qn, kn, v3, d(pos), d(cos), d(sin), kcd, vcd, d(slots))
+    if fused:   # q/k norm + rope + cache write in one launch
+        oq = F.rope_reshape_and_cache(q.reshape(B, Hq, D).contiguous(), k.reshape(B, Hkv, D).contiguous(), v3, d(pos),
+                                      d(cos), d(sin), kcd, vcd, d(slots), q_norm_weight=d(w_qn), k_norm_weight=d(w_kn),
+                                      epsilon=eps)
     else:
+        zq = torch.zeros(B * Hq, D, dtype=H, device=dev)
+        zk = torch.zeros(B * Hkv, D, dtype=H, device=dev)
+        qn = ops.add_rms_norm(q.reshape(B * Hq, D).contiguous(), zq, d(w_qn), eps)[0].view(B, Hq, D)
+        kn = ops.add_rms_norm(k.reshape(B * Hkv, D).contiguous(), zk, d(w_kn), eps)[0].view(B, Hkv, D)
         oq, ok = ops.rope(qn, kn, d(pos), d(cos), d(sin))
         ops.reshape_and_cache(ok, v3, kcd, vcd, d(slots))
     attn = ops.paged_attention(oq, kcd, vcd, d(bt), d(ctx))

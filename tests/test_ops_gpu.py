@@ -204,6 +204,48 @@ def test_rope_reshape_and_cache_fused_equals_the_chain(ops, dev, B, Hq, Hkv, D, 
     assert torch.equal(kc_b.cpu(), kc_ref) and torch.equal(vc_b.cpu(), vc_ref)
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,D,NB,P", [(64, 32, 8, 128, 2304, 128), (5, 6, 2, 64, 7, 16), (3, 1, 1, 16, 4, 8), (9, 4, 4, 256, 9, 32), (7, 3, 1, 32, 5, 4)])
+def test_qknorm_rope_reshape_and_cache_fused(ops, dev, B, Hq, Hkv, D, NB, P):
+    """Per-head RMSNorm of q and k + rope + cache write in one launch, against the oracle (RMSNorm rounded to fp16,
+    then rotated) and against the chain of separate device operators where those take the shape."""
+    import ascend910a_extras.fused as fused
+    g = _gen(8)
+    q = torch.randn(B, Hq, D, generator=g).half()
+    k = torch.randn(B, Hkv, D, generator=g).half()
+    v = torch.randn(B, Hkv, D, generator=g).half()
+    wq = (1 + 0.2 * torch.randn(D, generator=g)).half()
+    wk = (1 + 0.2 * torch.randn(D, generator=g)).half()
+    eps = 1e-6
+    cos, sin = R.build_cos_sin_cache(512, D, theta=1e6)
+    pos = torch.randint(0, 512, (B,), generator=g).int()
+    slots = torch.randperm(NB * P, generator=g)[:B].int()
+    kc0 = torch.randn(NB, Hkv * D // 16, P, 16, generator=g).half()
+    vc0 = torch.randn(NB, Hkv * D // 16, P, 16, generator=g).half()
+    qd, kd, vd, posd, cosd, sind, sld = (t.to(dev) for t in (q, k, v, pos, cos, sin, slots))
+    kcd, vcd = kc0.to(dev), vc0.to(dev)
+    oq, ok = fused.rope_reshape_and_cache(qd, kd, vd, posd, cosd, sind, kcd, vcd, sld, return_k=True,
+                                          q_norm_weight=wq.to(dev), k_norm_weight=wk.to(dev), epsilon=eps)
+
+    def rms(t, w):
+        t = t.float()
+        return (t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps) * w.float()).half()
+
+    rq, rk = R.rope_ref(rms(q, wq), rms(k, wk), pos, cos, sin)
+    torch.testing.assert_close(oq.cpu().float(), rq.float(), **TOL)
+    torch.testing.assert_close(ok.cpu().float(), rk.float(), **TOL)
+    # the caches hold exactly the rotated k the kernel reports, and v untouched
+    kc_ref, vc_ref = kc0.clone(), vc0.clone()
+    R.reshape_and_cache_ref(ok.cpu(), kc_ref, slots, v, vc_ref)
+    assert torch.equal(kcd.cpu(), kc_ref) and torch.equal(vcd.cpu(), vc_ref)
+    if D % 64 == 0:   # the separate RMSNorm operator takes rows that are multiples of 64
+        zq = torch.zeros(B * Hq, D, dtype=H, device=dev); zk = torch.zeros(B * Hkv, D, dtype=H, device=dev)
+        qn = ops.add_rms_norm(qd.view(B * Hq, D), zq, wq.to(dev), eps)[0].view(B, Hq, D)
+        kn = ops.add_rms_norm(kd.view(B * Hkv, D), zk, wk.to(dev), eps)[0].view(B, Hkv, D)
+        cq, ck = ops.rope(qn, kn, posd, cosd, sind)
+        torch.testing.assert_close(oq.float(), cq.float(), rtol=2e-3, atol=2e-3)
+        torch.testing.assert_close(ok.float(), ck.float(), rtol=2e-3, atol=2e-3)
+
+
 # ----------------------------------------------------------------------------- grouped_matmul
 def _gmm_case(rows, K, N, E, seed, counts=None, wstd=0.02):
     g = _gen(seed)
