@@ -1167,17 +1167,18 @@ static int aops_grouped_matmul_impl(const void* x, const void* w, const int64_t*
   const f16* xp = static_cast<const f16*>(x);
   const f16* wp = static_cast<const f16*>(w);
   f16* yp = static_cast<f16*>(y);
-  const char* forced_env = getenv("AOPS_GMM_VARIANT");  // tuning aid: 1..6 force one kernel / tile shape
+  const char* forced_env = getenv("AOPS_GMM_VARIANT");  // tuning aid: 1..8 force one kernel / tile shape
   const int forced = forced_env ? atoi(forced_env) : 0;
   // Tile choice from what the host knows (group_list stays on the device): the largest tile
   // whose grid still gives every CU work.  320 rows cover a typical expert of a large routed
   // batch in one tile; small or dense problems (few rows, one expert) take smaller tiles so that
   // enough workgroups exist to pull the weights through all memory channels.
   int variant = forced;
-  if (variant < 1 || variant > 6) {
+  if (variant < 1 || variant > 8) {
     auto tiles = [&](int64_t bm, int64_t bn) { return ((rows + bm - 1) / bm) * ((n + bn - 1) / bn); };
     constexpr int64_t kEnough = 384;
-    variant = tiles(320, 256) >= kEnough ? 6 : tiles(320, 128) >= kEnough ? 2 : tiles(256, 128) >= kEnough ? 3
+    constexpr int64_t kMostCus = 192;  // 256-row tiles read a small batch's weights once: worth a few idle CUs
+    variant = tiles(320, 256) >= kEnough ? 6 : tiles(320, 128) >= kEnough ? 2 : tiles(256, 128) >= kMostCus ? 3
               : tiles(128, 128) >= kEnough ? 4 : 5;
   }
   if (variant == 6 && (k % 128 != 0 || k < 256)) variant = 1;  // the persistent kernel's k loop
@@ -1185,6 +1186,10 @@ static int aops_grouped_matmul_impl(const void* x, const void* w, const int64_t*
     case 6:  // 320 x 256 tiles, eight waves, one persistent workgroup per CU
       return gmm_persistent_launch<5, 2, 4, false>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts,
                                             (int)n, s);
+    case 7:  // 256 x 128 tiles, four waves, operands copied HBM -> LDS directly
+      return gmm_dma_launch<4, 2, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
+    case 8:  // 128 x 128 tiles, four waves, operands copied HBM -> LDS directly
+      return gmm_dma_launch<2, 2, 2>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n, s);
     case 1:  // 320 x 256 tiles, eight waves, operands copied HBM -> LDS directly
       return gmm_dma_launch<5, 2, 4>(xp, wp, group_list, yp, rows, (int)k, (int)num_experts, (int)n,
                                      s);

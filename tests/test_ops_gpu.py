@@ -306,7 +306,7 @@ def test_grouped_matmul_does_not_write_past_the_last_group(ops, dev):
     torch.testing.assert_close(y.cpu()[:110].float(), ref[:110].float(), **GMM_TOL)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize(
     "rows,K,N,E,counts",
     [
@@ -318,7 +318,7 @@ def test_grouped_matmul_does_not_write_past_the_last_group(ops, dev):
 )
 def test_grouped_matmul_every_kernel(ops, dev, monkeypatch, variant, rows, K, N, E, counts):
     """The tile shape / kernel is normally chosen from the problem size; AOPS_GMM_VARIANT forces one,
-    so that every kernel sees the edge cases (6 = persistent kernel, needs K % 128 == 0, K >= 256)."""
+    so that every kernel sees the edge cases (6 = persistent kernel, needs K % 128 == 0, K >= 256; 7, 8 = direct-copy kernels with smaller tiles)."""
     import ascend910a_extras.ascend910a_extras_C as C
     monkeypatch.setenv("AOPS_GMM_VARIANT", str(variant))
     x, w, gl = _gmm_case(rows, K, N, E, seed=variant, counts=counts)
