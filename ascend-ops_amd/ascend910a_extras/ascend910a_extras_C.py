@@ -44,6 +44,8 @@ _SIGNATURES = {
     "aops_grouped_matmul_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_matmul_nt_f16": (ctypes.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
     "aops_grouped_matmul_swiglu_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
+    "aops_grouped_matmul_swiglu_gather_f16": (
+        ctypes.c_int, [_vp, _vp, _i64, _i64, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_moe_sort_workspace": (_sz, [_i64, _i64]),
     "aops_moe_sort_i32": (ctypes.c_int, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
     "aops_moe_gather_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
@@ -460,6 +462,35 @@ def rope_reshape_and_cache(q, k, v, position_ids, cos_cache, sin_cache, key_cach
     )
     _status(name, code)
     return [out_q, out_k] if return_k else out_q
+
+
+def grouped_matmul_swiglu_gather(x, sorted_idx, topk, w, group_list):
+    """grouped_matmul_swiglu(moe_gather(x, sorted_idx, group_list, topk), w, group_list) without the gathered
+    copy: the kernel reads row ``sorted_idx[j] // topk`` of ``x`` for sorted row ``j``."""
+    name = "grouped_matmul_swiglu_gather"
+    _check(x.dim() == 2 and x.is_contiguous() and sorted_idx.dim() == 1 and sorted_idx.is_contiguous(),
+           f"{name}: x must be 2D, sorted_idx 1D, both contiguous")
+    _check(topk > 0 and sorted_idx.numel() == x.size(0) * topk,
+           f"{name}: sorted_idx must have tokens*topk entries, got {sorted_idx.numel()} for {x.size(0)} tokens, topk {topk}")
+    rows = sorted_idx.numel()
+    dim = x.size(1)
+    if dim % 128 != 0 or dim < 256 or x.size(0) * dim >= 2 ** 32:
+        return grouped_matmul_swiglu(moe_gather(x, sorted_idx, group_list, topk), w, group_list)
+    # the remaining checks are those of grouped_matmul on the (virtual) gathered matrix
+    _check(w.dim() == 3 and group_list.dim() == 1 and group_list.is_contiguous(), f"{name}: w must be 3D, group_list 1D")
+    _check(dim == w.size(1), f"{name}: last dimension of x must match second dimension of w, got {dim} and {w.size(1)}")
+    _check(w.stride(1) == 1 and w.stride(2) == dim, f"{name}: w must be K-major order, got strides {tuple(w.stride())}")
+    _check(w.size(2) % 64 == 0, f"{name}: third dimension of w must be a multiple of 64, got {w.size(2)}")
+    num_experts, inner_dim = w.size(0), w.size(2)
+    _check(num_experts <= 1 or w.stride(0) == dim * inner_dim, f"{name}: experts of w must be densely packed")
+    _check(group_list.size(0) == num_experts, f"{name}: group_list must have one entry per expert")
+    _require_device(name, {"x": (x, torch.float16), "w": (w, torch.float16), "group_list": (group_list, torch.int64),
+                           "sorted_idx": (sorted_idx, torch.int32)})
+    y = torch.empty((rows, inner_dim // 2), dtype=x.dtype, device=x.device)
+    code = _lib.aops_grouped_matmul_swiglu_gather_f16(_ptr(x), _ptr(sorted_idx), topk, x.size(0), _ptr(w), _ptr(group_list),
+                                                      _ptr(y), rows, dim, num_experts, inner_dim, _stream(x.device))
+    _status(name, code)
+    return y
 
 
 def moe_sort(topk_ids, num_experts):

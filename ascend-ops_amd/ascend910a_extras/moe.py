@@ -30,10 +30,10 @@ def moe_mlp(x: torch.Tensor, topk_ids: torch.Tensor, topk_weights: torch.Tensor,
             w_down: torch.Tensor) -> torch.Tensor:
     """Expert MLP of a routed batch: ``x`` ``[tokens, hidden]`` fp16, ``topk_ids`` int32 and ``topk_weights``
     fp32 ``[tokens, topk]``, ``w_gate_up`` logical ``[E, hidden, 2*inter]`` and ``w_down`` logical
-    ``[E, inter, hidden]`` in the layout of ``ops.grouped_matmul``.  Five launches, no host round trip."""
+    ``[E, inter, hidden]`` in the layout of ``ops.grouped_matmul``.  The row gather happens inside the first
+    grouped matmul's operand copies, the activation in its epilogue; no host round trip."""
     num_experts = w_gate_up.size(0)
     sorted_idx, inverse_idx, group_list = moe_sort(topk_ids, num_experts)
-    xs = moe_gather(x, sorted_idx, group_list, topk_ids.size(1))
-    act = _C.grouped_matmul_swiglu(xs, w_gate_up, group_list)
+    act = _C.grouped_matmul_swiglu_gather(x, sorted_idx, topk_ids.size(1), w_gate_up, group_list)
     y = _C.grouped_matmul(act, w_down, group_list)
     return moe_combine(y, inverse_idx, topk_weights, topk_ids, num_experts)

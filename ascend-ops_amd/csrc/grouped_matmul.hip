@@ -754,10 +754,16 @@ __device__ __forceinline__ GmmWork gmm_locate(const GmmPlan& p,
 // column wn, the 32 gate rows of its columns in row block 2*wn and the matching 32 up rows in row
 // block 2*wn + 1, so that a lane finds gate and up value of one output element in acc[i][0] and
 // acc[i][1].
-template <int MB, int NB, int WN, bool SWIGLU>
+//
+// GATHER = true reads the activation rows through an index: sorted row j comes from row
+// row_idx[j] / idx_div of x (the routing order of a mixture of experts: row_idx = the sorted flat
+// routing indices, idx_div = top-k), so the expert-sorted copy of x never exists.  The tile's
+// source rows are looked up once per work item.
+template <int MB, int NB, int WN, bool SWIGLU, bool GATHER>
 __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kernel(
     const f16* __restrict__ x, const f16* __restrict__ w, const int64_t* __restrict__ group_list,
-    f16* __restrict__ y, int64_t rows, int k, int num_experts, int n) {
+    f16* __restrict__ y, int64_t rows, int k, int num_experts, int n,
+    const int32_t* __restrict__ row_idx, int idx_div, uint32_t x_rows) {
   constexpr int kWaves = 2 * WN;
   constexpr int BM = 64 * MB;
   constexpr int BN = 32 * NB * WN;
@@ -833,15 +839,27 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   const uint32_t off0 = (uint32_t)lane_row * (uint32_t)k + lane_c * 8;
   const uint32_t copy_stride = 8u * kWaves * (uint32_t)k;
   uint32_t a_last, b_last;  // offset of this lane's chunk in the last valid row
+  uint32_t a_src[GATHER ? kACopies : 1];  // GATHER: offset of this lane's chunk per copy
   // SWIGLU: copy i of the weights fills row blocks 2i (gate rows 32i..32i+31 of the item) and
   // 2i+1 (the up rows d further down): per-lane offset + 32 rows per copy; b_last then holds the
   // number of valid 32-column blocks of the item instead of an offset.
   const uint32_t off0_glu = ((uint32_t)(lane_row & 31) + (lane_row >= 32 ? (uint32_t)n_out : 0u)) * (uint32_t)k + lane_c * 8;
   auto set_sources = [&](const GmmWork& it) {
-    a_base = x + (int64_t)it.row_begin * k;
     b_base = w + ((int64_t)it.expert * n + (int64_t)it.n_tile * BNO) * k;
     const int n_left = min(n_out - it.n_tile * BNO, BNO);
     const int x_left = min(it.row_end - it.row_begin, BM);  // rows of the group in this tile
+    if constexpr (GATHER) {
+      a_base = x;
+#pragma unroll
+      for (int i = 0; i < kACopies; ++i) {
+        const int r = min(8 * kWaves * i + lane_row, x_left - 1);
+        uint32_t src = (uint32_t)row_idx[it.row_begin + r] / (uint32_t)idx_div;
+        src = src < x_rows ? src : x_rows - 1;  // an index outside x reads its last row instead of faulting
+        a_src[i] = src * (uint32_t)k + lane_c * 8;
+      }
+    } else {
+      a_base = x + (int64_t)it.row_begin * k;
+    }
     a_last = (uint32_t)(x_left - 1) * (uint32_t)k + lane_c * 8;
     b_last = SWIGLU ? (uint32_t)(n_left / 32) : (uint32_t)(n_left - 1) * (uint32_t)k + lane_c * 8;
   };
@@ -857,14 +875,22 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     const int ko = kt * kBK;
     f16* da = sa + stage * BM * kBK + wave * 512;
     f16* db = sb + stage * BN * kBK + wave * 512;
+    // the empty asm makes the 64-bit source address of a copy be formed right before the copy
+    // instead of being kept in a register pair per copy across the k loop
 #pragma unroll
-    for (int i = 0; i < kACopies; ++i)
-      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(a_base + ko + min(off0 + i * copy_stride, a_last)),
+    for (int i = 0; i < kACopies; ++i) {
+      uint32_t o = GATHER ? a_src[i] : min(off0 + i * copy_stride, a_last);
+      asm volatile("" : "+v"(o));
+      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(a_base + ko + o),
                                        AOPS_LDS_PTR(da + i * kWaves * 512), 16, 0, 0);
+    }
 #pragma unroll
-    for (int i = 0; i < kBCopies; ++i)
-      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(b_base + ko + b_offset(i)),
+    for (int i = 0; i < kBCopies; ++i) {
+      uint32_t o = b_offset(i);
+      asm volatile("" : "+v"(o));
+      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(b_base + ko + o),
                                        AOPS_LDS_PTR(db + i * kWaves * 512), 16, 0, 0);
+    }
   };
 
   const int fm = lane & 31;
@@ -1058,9 +1084,10 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
 }
 
-template <int MB, int NB, int WN, bool SWIGLU>
+template <int MB, int NB, int WN, bool SWIGLU, bool GATHER = false>
 static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* group_list, f16* y,
-                                 int64_t rows, int k, int num_experts, int n, hipStream_t stream) {
+                                 int64_t rows, int k, int num_experts, int n, hipStream_t stream,
+                                 const int32_t* row_idx = nullptr, int idx_div = 1, int64_t x_rows = 1) {
   constexpr int BM = 64 * MB;
   constexpr int BN = 32 * NB * WN;
   constexpr int kWaves = 2 * WN;
@@ -1084,7 +1111,7 @@ static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* grou
   int64_t grid = cus[dev] < max_work ? cus[dev] : max_work;
   grid = grid / kXcds * kXcds;
   if (grid < kXcds) grid = kXcds;
-  auto kernel = grouped_matmul_persistent_kernel<MB, NB, WN, SWIGLU>;
+  auto kernel = grouped_matmul_persistent_kernel<MB, NB, WN, SWIGLU, GATHER>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -1093,7 +1120,7 @@ static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* grou
     attr_set = true;
   }
   kernel<<<(unsigned)grid, 2 * WN * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts,
-                                                          n);
+                                                          n, row_idx, idx_div, (uint32_t)x_rows);
   return record_launch_status(hipGetLastError());
 }
 
@@ -1234,4 +1261,24 @@ extern "C" int aops_matmul_nt_f16(const void* x, const void* w, void* y, int64_t
   if (m == 0) return AOPS_OK;
   if (!x || !w || !y) return AOPS_ERR_INVALID_ARGUMENT;
   return aops_grouped_matmul_impl(x, w, nullptr, y, m, k, 1, n, stream);
+}
+
+extern "C" int aops_grouped_matmul_swiglu_gather_f16(const void* x, const int32_t* row_idx,
+                                                     int64_t idx_div, int64_t x_rows, const void* w,
+                                                     const int64_t* group_list, void* y, int64_t rows,
+                                                     int64_t k, int64_t num_experts, int64_t n,
+                                                     void* stream) {
+  using namespace aops;
+  if (rows < 0 || k <= 0 || n <= 0 || num_experts < 0 || k % 128 != 0 || k < 256 || n % 64 != 0 ||
+      idx_div <= 0 || idx_div > 0x7fffffff || x_rows < 0 || (rows > 0 && x_rows == 0))
+    return AOPS_ERR_INVALID_ARGUMENT;
+  // 32-bit per-lane offsets: x_rows activation rows and (n/2 + 32) weight rows of k elements must fit
+  if (rows > 0x7fffffff - 4096 || k > (1 << 22) || n > 0x7fffffff || num_experts > (1 << 20) ||
+      (n / 2 + 320) * k > 0x7fffffffLL || x_rows * k > 0xffffffffLL)
+    return AOPS_ERR_INVALID_ARGUMENT;
+  if (rows == 0 || num_experts == 0) return AOPS_OK;
+  if (!x || !row_idx || !w || !group_list || !y) return AOPS_ERR_INVALID_ARGUMENT;
+  return gmm_persistent_launch<5, 2, 4, true, true>(
+      static_cast<const f16*>(x), static_cast<const f16*>(w), group_list, static_cast<f16*>(y), rows,
+      (int)k, (int)num_experts, (int)n, static_cast<hipStream_t>(stream), row_idx, (int)idx_div, x_rows);
 }

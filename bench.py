@@ -347,6 +347,35 @@ def _gmm_swiglu_entry(L, ops, dev, config, x, w_storage, gl, h_dev):
     return e
 
 
+def _gmm_swiglu_gather_entry(L, dev, w_storage, tokens, topk):
+    """Fused gate_up + SwiGLU that also reads its rows through the routing order (extension): x stays in token
+    order [tokens, hidden]; checked bit for bit against the explicit gather followed by the fused kernel."""
+    import torch
+    import ascend910a_extras.ascend910a_extras_C as C
+    import ascend910a_extras.moe as moe
+
+    E, N, K = w_storage.shape
+    rows = tokens * topk
+    torch.manual_seed(2)
+    ids = torch.randint(0, E, (tokens, topk), dtype=torch.int32).to(dev)
+    x = torch.randn(tokens, K).half().to(dev)
+    wd = w_storage.to(dev)
+    s_idx, _, gl = moe.moe_sort(ids, E)
+    flops = 2 * rows * K * N
+    alg = tokens * K * 2 + E * N * K * 2 + rows * (N // 2) * 2 + rows * 4 + E * 8
+    y = torch.empty(rows, N // 2, dtype=torch.float16, device=dev)
+    call = lambda: L.check(L.lib.aops_grouped_matmul_swiglu_gather_f16(x.data_ptr(), s_idx.data_ptr(), topk, tokens,
+                                                                       wd.data_ptr(), gl.data_ptr(), y.data_ptr(), rows, K, E, N,
+                                                                       L.stream()))
+    med, mn = time_graph([call], min_launches=40)
+    want = C.grouped_matmul_swiglu(moe.moe_gather(x, s_idx, gl, topk), wd.transpose(1, 2), gl)
+    assert torch.equal(y, want)
+    return entry("grouped_matmul_swiglu_gather", "4: MoE gate_up + activation + row gather, fused",
+                 f"x [{tokens},{K}] (token order, top-{topk}) @ w [{E},{K},{N}] f16 -> [{rows},{N // 2}]", "mfma", alg, flops,
+                 med, mn, None, None, 1,
+                 "extension: replaces moe_gather + gate_up + swiglu; one weight set, so the weights are re-read from HBM every launch but x (17 MB) stays cached")
+
+
 def _moe_glue_entries(L, dev, E, hidden, tokens, topk):
     """Routing glue of the expert MLP at the configs[3] shape (extension, no reference operator): device-side
     stable sort -> group_list, row gather, weighted combine.  Checked against the oracle in tests/test_moe_gpu.py."""
@@ -405,6 +434,7 @@ def bench_moe(L, ops, R, dev, cpu):
     e1, h_dev = _gmm_entry(L, ops, R, dev, cpu, "grouped_matmul", "4: MoE gate_up", x, w1, gl)
     out.append(e1)
     e_fused = _gmm_swiglu_entry(L, ops, dev, "4: MoE gate_up + activation, fused", x, w1, gl, h_dev)
+    e_gather = _gmm_swiglu_gather_entry(L, dev, w1, tokens, topk)
     del w1
     h = ops.swiglu(h_dev)
     # swiglu at the MoE shape
@@ -424,6 +454,7 @@ def bench_moe(L, ops, R, dev, cpu):
     e2, _ = _gmm_entry(L, ops, R, dev, cpu, "grouped_matmul", "4: MoE down", h.cpu(), w2, gl)
     out.append(e2)
     out.append(e_fused)
+    out.append(e_gather)
     out.extend(_moe_glue_entries(L, dev, E, hidden, tokens, topk))
     tot_flops = e1["algorithmic_flops"] + e2["algorithmic_flops"]
     tot_us = e1["gpu_us"] + e2["gpu_us"]

@@ -163,6 +163,17 @@ int aops_grouped_matmul_swiglu_f16(const void* x, const void* w, const int64_t* 
                                    void* stream);
 
 /*
+ * aops_grouped_matmul_swiglu_f16 with the row gather of a routed batch folded into the operand
+ * copies: sorted row j is row row_idx[j] / idx_div of x (x: [x_rows, k]; row_idx: int32 [rows], e.g.
+ * sorted_idx of aops_moe_sort_i32 with idx_div = top-k), so the expert-sorted copy of x is never
+ * written.  y: [rows, n/2].  Same shape limits; x_rows * k must be below 2^32.
+ */
+int aops_grouped_matmul_swiglu_gather_f16(const void* x, const int32_t* row_idx, int64_t idx_div,
+                                          int64_t x_rows, const void* w, const int64_t* group_list,
+                                          void* y, int64_t rows, int64_t k, int64_t num_experts,
+                                          int64_t n, void* stream);
+
+/*
  * Routing glue of an expert MLP (no counterpart among the reference's operators: its caller does
  * these steps; the reference itself only shows the host-side construction of group_list,
  * benchmark/test_grouped_matmul.py:46-50).

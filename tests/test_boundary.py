@@ -92,6 +92,10 @@ def test_c_abi_rejects_bad_sizes_without_touching_the_gpu():
     assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 128, 2, 128, None) == -1   # k < 256
     assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 256, 2, 128, None) == -1   # null pointers
     assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 0, 256, 2, 128, None) == 0
+    assert lib.aops_grouped_matmul_swiglu_gather_f16(None, None, 8, 16, None, None, None, 128, 192, 2, 128, None) == -1  # k % 128
+    assert lib.aops_grouped_matmul_swiglu_gather_f16(None, None, 0, 16, None, None, None, 128, 256, 2, 128, None) == -1  # divisor
+    assert lib.aops_grouped_matmul_swiglu_gather_f16(None, None, 8, 16, None, None, None, 128, 256, 2, 128, None) == -1  # null pointers
+    assert lib.aops_grouped_matmul_swiglu_gather_f16(None, None, 8, 16, None, None, None, 0, 256, 2, 128, None) == 0
     n = [None] * 11
     assert lib.aops_rope_reshape_and_cache_f16(*n, 2, 4, 2, 24, 8, 16, None) == -1                   # head_dim % 16
     assert lib.aops_rope_reshape_and_cache_f16(*n, 2, 4, 2, 64, 8, 16, None) == -1                   # null pointers

@@ -81,3 +81,22 @@ def test_moe_mlp_end_to_end(dev, tokens, topk, E, hidden, inter):
     ref = R.moe_mlp_ref(x, ids, wts, w1, w2)
     assert out.shape == (tokens, hidden) and out.dtype == H
     torch.testing.assert_close(out.cpu().float(), ref, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("tokens,topk,E,hidden,inter", [(700, 4, 16, 256, 128), (4096, 8, 128, 512, 384), (50, 2, 300, 384, 64)])
+def test_gather_fused_gate_up_equals_gather_then_matmul(dev, tokens, topk, E, hidden, inter):
+    """The grouped matmul that reads its rows through the routing order against the explicit gather followed by the
+    same kernel without the index: bit for bit (same arithmetic, same order), invalid ids included."""
+    import ascend910a_extras.ascend910a_extras_C as C
+    import ascend910a_extras.moe as moe
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(tokens, hidden, generator=g).half().to(dev)
+    ids = torch.randint(0, E, (tokens, topk), generator=g, dtype=torch.int32)
+    ids[torch.rand(tokens, topk, generator=g) < 0.05] = -1
+    w1 = (torch.randn(E, 2 * inter, hidden, generator=g) / hidden ** 0.5).half().to(dev).transpose(1, 2)
+    s, inv, gl = moe.moe_sort(ids.to(dev), E)
+    end = int(gl[-1])
+    a = C.grouped_matmul_swiglu_gather(x, s, topk, w1, gl)
+    b = C.grouped_matmul_swiglu(moe.moe_gather(x, s, gl, topk), w1, gl)
+    assert a.shape == (tokens * topk, inter)
+    assert torch.equal(a[:end], b[:end])
