@@ -119,10 +119,20 @@ __global__ __launch_bounds__(1024) void moe_scan_kernel(int32_t* __restrict__ co
   }
 }
 
+// SCAN = false: counts holds the exclusive prefixes over the slices and base the exclusive prefix
+// over the buckets (moe_scan_kernel ran).  SCAN = true (few slices, at most kFoldBuckets buckets):
+// counts holds the raw histograms and every wave derives its own starting positions from them -
+// the per-bucket sum over the earlier slices and the exclusive scan of the bucket totals - which
+// saves the scan kernel's launch; the wave of slice 0 writes group_list.
+constexpr int kFoldSlices = 128;
+constexpr int kFoldBuckets = 256;
+
+template <bool SCAN>
 __global__ __launch_bounds__(kMoeWaves* kWave) void moe_scatter_kernel(
     const int32_t* __restrict__ ids, int64_t n, int num_experts, int num_slices,
     const int32_t* __restrict__ counts, const int32_t* __restrict__ base,
-    int32_t* __restrict__ sorted_idx, int32_t* __restrict__ inverse_idx, int id_bits) {
+    int32_t* __restrict__ sorted_idx, int32_t* __restrict__ inverse_idx, int id_bits,
+    int64_t* __restrict__ group_list) {
   extern __shared__ int32_t run_lds[];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
@@ -130,8 +140,47 @@ __global__ __launch_bounds__(kMoeWaves* kWave) void moe_scatter_kernel(
   const int buckets = num_experts + 1;
   int32_t* running = run_lds + wave * buckets;
   if (slice >= num_slices) return;  // wave uniform; no workgroup barrier below
-  const int32_t* mine = counts + (int64_t)slice * buckets;
-  for (int e = lane; e < buckets; e += kWave) running[e] = base[e] + mine[e];
+  if constexpr (SCAN) {
+    constexpr int kPer = kFoldBuckets / kWave;  // bucket e = lane + 64*j
+    int before[kPer], total[kPer];
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) before[j] = total[j] = 0;
+    for (int s0 = 0; s0 < num_slices; s0 += 8) {  // eight rows of loads in flight
+      int c[8][kPer];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+          const int e = lane + kWave * j;
+          c[u][j] = (s0 + u < num_slices && e < buckets) ? counts[(int64_t)(s0 + u) * buckets + e] : 0;
+        }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+          total[j] += c[u][j];
+          if (s0 + u < slice) before[j] += c[u][j];
+        }
+    }
+    int carry = 0;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      int incl = total[j];
+#pragma unroll
+      for (int d = 1; d < kWave; d <<= 1) {
+        const int up = __shfl_up(incl, d);
+        if (lane >= d) incl += up;
+      }
+      const int excl = carry + incl - total[j];
+      carry += __shfl(incl, kWave - 1);
+      const int e = lane + kWave * j;
+      if (e < buckets) running[e] = excl + before[j];
+      if (slice == 0 && e < num_experts) group_list[e] = (int64_t)excl + total[j];
+    }
+  } else {
+    const int32_t* mine = counts + (int64_t)slice * buckets;
+    for (int e = lane; e < buckets; e += kWave) running[e] = base[e] + mine[e];
+  }
   const int64_t begin = (int64_t)slice * kSlice;
   const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
   int idv[kSlice / kWave];  // all loads first: one memory latency per slice instead of eight
@@ -248,6 +297,8 @@ extern "C" int aops_moe_sort_i32(const int32_t* expert_ids, int64_t n, int64_t n
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int slices = (int)moe_slices(n);
   const int buckets = (int)num_experts + 1;
+  int id_bits = 1;  // bits needed for bucket numbers 0..num_experts
+  while ((1 << id_bits) <= (int)num_experts) ++id_bits;
   int32_t* counts = static_cast<int32_t*>(workspace);           // [slices][E+1]
   int32_t* base = counts + (int64_t)slices * buckets;           // [E+1]
   const size_t lds = (size_t)kMoeWaves * buckets * sizeof(int32_t);
@@ -257,14 +308,19 @@ extern "C" int aops_moe_sort_i32(const int32_t* expert_ids, int64_t n, int64_t n
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return record_launch_status(e);
   }
+  if (slices > 0 && slices <= kFoldSlices && buckets <= kFoldBuckets) {  // two launches
+    moe_scatter_kernel<true><<<grid, kMoeWaves * kWave, lds, s>>>(expert_ids, n, (int)num_experts, slices,
+                                                                 counts, base, sorted_idx, inverse_idx,
+                                                                 id_bits, group_list);
+    return record_launch_status(hipGetLastError());
+  }
   moe_scan_kernel<<<1, 1024, 0, s>>>(counts, slices, (int)num_experts, base, group_list);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return record_launch_status(e);
   if (slices > 0) {
-    int id_bits = 1;  // bits needed for bucket numbers 0..num_experts
-    while ((1 << id_bits) <= (int)num_experts) ++id_bits;
-    moe_scatter_kernel<<<grid, kMoeWaves * kWave, lds, s>>>(expert_ids, n, (int)num_experts, slices, counts,
-                                                           base, sorted_idx, inverse_idx, id_bits);
+    moe_scatter_kernel<false><<<grid, kMoeWaves * kWave, lds, s>>>(expert_ids, n, (int)num_experts, slices,
+                                                                  counts, base, sorted_idx, inverse_idx,
+                                                                  id_bits, group_list);
     e = hipGetLastError();
   }
   return record_launch_status(e);
