@@ -30,6 +30,8 @@ SOURCES = [
     "reshape_and_cache.hip",
     "paged_attention.hip",
     "grouped_matmul.hip",
+    "grouped_matmul_tiles.hip",
+    "grouped_matmul_persistent.hip",
 ]
 
 # -packed-fp32-ops: keep the compiler from forming packed-fp32 VALU instructions.

@@ -1,0 +1,402 @@
+// Grouped matmul, persistent kernel for large problems (optionally with the SwiGLU activation in
+// the epilogue and the row gather of a routed batch in the operand copies).
+#include "gmm_common.h"
+
+namespace aops {
+
+// Persistent form of grouped_matmul_dma_kernel: one workgroup per CU walks through its share of
+// the work items (XCD x owns a contiguous range of items, its workgroups take them round robin),
+// and the operand pipeline never drains between items: the last two k tiles of an item issue the
+// copies of the first two tiles of the next item, and the finished accumulators leave straight
+// from registers (lane pairs exchange halves with v_permlane32_swap so that every lane stores 16
+// contiguous bytes) while those copies are in flight, with no LDS use and no workgroup barrier.
+// group_list is scanned once per workgroup; every wave keeps its copy of the scan in LDS.
+// Requires k % 128 == 0 and k >= 256 (an even number of k tiles keeps the stage parity fixed).
+//
+// SWIGLU = true fuses the activation of a gate_up projection into the epilogue: with d = n/2 the
+// kernel writes y[r, c] = silu(h[r, c]) * h[r, d + c] (h = x @ W_e^T in fp32, never stored) as a
+// [rows, d] matrix.  A work item then covers 32*WN output columns; the weight stage holds, for wave
+// column wn, the 32 gate rows of its columns in row block 2*wn and the matching 32 up rows in row
+// block 2*wn + 1, so that a lane finds gate and up value of one output element in acc[i][0] and
+// acc[i][1].
+//
+// GATHER = true reads the activation rows through an index: sorted row j comes from row
+// row_idx[j] / idx_div of x (the routing order of a mixture of experts: row_idx = the sorted flat
+// routing indices, idx_div = top-k), so the expert-sorted copy of x never exists.  The tile's
+// source rows are looked up once per work item.
+template <int MB, int NB, int WN, bool SWIGLU, bool GATHER>
+__global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kernel(
+    const f16* __restrict__ x, const f16* __restrict__ w, const int64_t* __restrict__ group_list,
+    f16* __restrict__ y, int64_t rows, int k, int num_experts, int n,
+    const int32_t* __restrict__ row_idx, int idx_div, uint32_t x_rows) {
+  constexpr int kWaves = 2 * WN;
+  constexpr int BM = 64 * MB;
+  constexpr int BN = 32 * NB * WN;
+  constexpr int kSteps = kBK / 16;
+  constexpr int kACopies = BM / 8 / kWaves;
+  constexpr int kBCopies = BN / 8 / kWaves;
+  static_assert(BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0, "tile rows per copy");
+  static_assert(!SWIGLU || (NB == 2 && kWaves == 8), "gate/up pairing assumes 64-row copies, two column blocks");
+  constexpr int BNO = SWIGLU ? BN / 2 : BN;  // output columns per work item
+  const int n_out = SWIGLU ? n / 2 : n;      // output row length
+
+  extern __shared__ __attribute__((aligned(16))) f16 smem[];
+  f16* sa = smem;                         // [2][BM * kBK]
+  f16* sb = smem + 2 * BM * kBK;          // [2][BN * kBK]
+  int* splan = reinterpret_cast<int*>(smem + 2 * (BM + BN) * kBK);  // [kWaves][kWave][8]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave / WN;
+  const int wn = wave % WN;
+  const int n_tiles = (n_out + BNO - 1) / BNO;
+  const int ktiles = k / kBK;
+
+  int* my_plan = splan + (wave * kWave + lane) * 8;
+  int plan_per, plan_total;
+  {
+    const GmmPlan plan = gmm_make_plan<BM>(group_list, num_experts, rows);
+    plan_per = __builtin_amdgcn_readfirstlane(plan.per);
+    plan_total = __builtin_amdgcn_readfirstlane(plan.total_tiles);
+    my_plan[0] = plan.tiles;
+    my_plan[1] = plan.incl;
+#pragma unroll
+    for (int j = 0; j <= kBndCache; ++j) my_plan[2 + j] = plan.bnd[j];
+  }
+  const int64_t total_work = (int64_t)plan_total * n_tiles;
+  const int64_t share = (total_work + kXcds - 1) / kXcds;
+  const int xcd = blockIdx.x % kXcds;
+  const int wg_in_xcd = blockIdx.x / kXcds;
+  const int wgs_per_xcd = gridDim.x / kXcds;
+  auto locate = [&](int64_t local) -> GmmWork {
+    const int64_t item = (int64_t)xcd * share + local;
+    if (local >= share || item >= total_work) {
+      GmmWork none;
+      none.valid = false;
+      none.expert = none.row_begin = none.row_end = none.n_tile = 0;
+      return none;
+    }
+    GmmPlan plan;  // this lane's part, written by this lane: no synchronisation needed
+    plan.per = plan_per;
+    plan.total_tiles = plan_total;
+    plan.tiles = my_plan[0];
+    plan.incl = my_plan[1];
+#pragma unroll
+    for (int j = 0; j <= kBndCache; ++j) plan.bnd[j] = my_plan[2 + j];
+    return gmm_locate<BM>(plan, group_list, num_experts, rows, n_tiles, item);
+  };
+
+  int64_t local = wg_in_xcd;
+  GmmWork cur = locate(local);
+  if (!cur.valid) return;
+
+  // Copy sources of the item whose tiles are being fetched.  Copy i of this wave fills physical
+  // rows (kWaves*i + wave)*8 .. +7 of a stage, i.e. logical row 8*kWaves*i + lane_row (the row
+  // swizzle only swaps rows inside the 8-row group) and chunk lane_c: one per-lane offset plus a
+  // uniform stride per copy, clamped to the last valid row: tile rows past the end of the group
+  // (only dead output rows depend on them) and past the end of w repeat the last valid row, which
+  // costs one cache line per copy instead of eight.
+  const f16* a_base;
+  const f16* b_base;
+  const int lane_row = wave * 8 + ((lane >> 3) ^ (wave & 1));
+  const int lane_c = (lane & 7) ^ (lane_row & 7);
+  const uint32_t off0 = (uint32_t)lane_row * (uint32_t)k + lane_c * 8;
+  const uint32_t copy_stride = 8u * kWaves * (uint32_t)k;
+  uint32_t a_last, b_last;  // offset of this lane's chunk in the last valid row
+  uint32_t a_src[GATHER ? kACopies : 1];  // GATHER: offset of this lane's chunk per copy
+  // SWIGLU: copy i of the weights fills row blocks 2i (gate rows 32i..32i+31 of the item) and
+  // 2i+1 (the up rows d further down): per-lane offset + 32 rows per copy; b_last then holds the
+  // number of valid 32-column blocks of the item instead of an offset.
+  const uint32_t off0_glu = ((uint32_t)(lane_row & 31) + (lane_row >= 32 ? (uint32_t)n_out : 0u)) * (uint32_t)k + lane_c * 8;
+  auto set_sources = [&](const GmmWork& it) {
+    b_base = w + ((int64_t)it.expert * n + (int64_t)it.n_tile * BNO) * k;
+    const int n_left = min(n_out - it.n_tile * BNO, BNO);
+    const int x_left = min(it.row_end - it.row_begin, BM);  // rows of the group in this tile
+    if constexpr (GATHER) {
+      a_base = x;
+#pragma unroll
+      for (int i = 0; i < kACopies; ++i) {
+        const int r = min(8 * kWaves * i + lane_row, x_left - 1);
+        uint32_t src = (uint32_t)row_idx[it.row_begin + r] / (uint32_t)idx_div;
+        src = src < x_rows ? src : x_rows - 1;  // an index outside x reads its last row instead of faulting
+        a_src[i] = src * (uint32_t)k + lane_c * 8;
+      }
+    } else {
+      a_base = x + (int64_t)it.row_begin * k;
+    }
+    a_last = (uint32_t)(x_left - 1) * (uint32_t)k + lane_c * 8;
+    b_last = SWIGLU ? (uint32_t)(n_left / 32) : (uint32_t)(n_left - 1) * (uint32_t)k + lane_c * 8;
+  };
+  auto b_offset = [&](int i) -> uint32_t {
+    if constexpr (SWIGLU) {
+      const uint32_t blk = (uint32_t)i < b_last ? (uint32_t)i : 0u;  // blocks past n: repeat block 0
+      return off0_glu + blk * 32u * (uint32_t)k;
+    } else {
+      return min(off0 + i * copy_stride, b_last);
+    }
+  };
+  auto copy_tile = [&](int kt, int stage) {
+    const int ko = kt * kBK;
+    f16* da = sa + stage * BM * kBK + wave * 512;
+    f16* db = sb + stage * BN * kBK + wave * 512;
+    // the empty asm makes the 64-bit source address of a copy be formed right before the copy
+    // instead of being kept in a register pair per copy across the k loop
+#pragma unroll
+    for (int i = 0; i < kACopies; ++i) {
+      uint32_t o = GATHER ? a_src[i] : min(off0 + i * copy_stride, a_last);
+      asm volatile("" : "+v"(o));
+      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(a_base + ko + o),
+                                       AOPS_LDS_PTR(da + i * kWaves * 512), 16, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < kBCopies; ++i) {
+      uint32_t o = b_offset(i);
+      asm volatile("" : "+v"(o));
+      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(b_base + ko + o),
+                                       AOPS_LDS_PTR(db + i * kWaves * 512), 16, 0, 0);
+    }
+  };
+
+  const int fm = lane & 31;
+  const int fq = lane >> 5;
+  // Fragment addresses: lds_off(fm, 2*st + fq) == lds_off(fm, fq) ^ (st << 4) (the k step only
+  // flips two chunk bits), so one per-lane offset per operand serves every k step.
+  const int fa_off0 = lds_off(fm, fq) + wm * 32 * kBK;
+  const int fb_off0 = lds_off(fm, fq) + wn * 32 * NB * kBK;
+
+  f32x16 acc[MB][NB];
+  GmmWork nxt;
+
+  auto k_loop = [&](auto live_c) {
+    constexpr int LIVE = decltype(live_c)::value;
+    f16x8 fa[2][LIVE > 0 ? LIVE : 1], fb[2][NB];
+    auto load_frags = [&](int buf, int st, int stage) {
+      // the empty asm keeps the compiler from hoisting one address register per (stage, step)
+      // out of the k loop, which would push the accumulators into scratch
+      int fo_a = fa_off0, fo_b = fb_off0;
+      asm volatile("" : "+v"(fo_a), "+v"(fo_b));
+      const f16* ca = sa + stage * BM * kBK + (fo_a ^ (st << 4));
+      const f16* cb = sb + stage * BN * kBK + (fo_b ^ (st << 4));
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        fb[buf][j] = *reinterpret_cast<const f16x8*>(&cb[j * 32 * kBK]);
+#pragma unroll
+      for (int i = 0; i < LIVE; ++i)
+        fa[buf][i] = *reinterpret_cast<const f16x8*>(&ca[i * 64 * kBK]);
+    };
+    auto step = [&](int kcopy, auto stage_c, auto st_c) {
+      constexpr int STAGE = decltype(stage_c)::value;
+      constexpr int ST = decltype(st_c)::value;
+      if (ST + 1 < kSteps) {
+        load_frags((ST + 1) & 1, ST + 1, STAGE);
+      } else {
+        load_frags(0, 0, STAGE ^ 1);  // first fragments of the next tile
+        copy_tile(kcopy, STAGE);      // this stage is free: everyone is past the barrier
+      }
+#pragma unroll
+      for (int i = 0; i < LIVE; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ST & 1][j], fa[ST & 1][i],
+                                                             acc[i][j], 0, 0, 0);
+      MfmaInterleave<0, LIVE * NB, LIVE + NB, 0,
+                     (ST + 1 < kSteps) ? 0 : kACopies + kBCopies>::run();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto iteration = [&](int kcopy, auto stage_c) {
+      step(kcopy, stage_c, std::integral_constant<int, 0>{});
+      step(kcopy, stage_c, std::integral_constant<int, 1>{});
+      step(kcopy, stage_c, std::integral_constant<int, 2>{});
+      // own copies of the next tile and all own fragment reads of this tile are complete ...
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();  // ... and so are everybody else's
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      step(kcopy, stage_c, std::integral_constant<int, 3>{});
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    load_frags(0, 0, 0);
+    for (int kt = 0; kt < ktiles; kt += 2) {
+      int c0 = kt + 2, c1 = kt + 3;
+      if (kt + 2 >= ktiles) {  // the last two tiles fetch the head of the next item
+        if (nxt.valid) {
+          set_sources(nxt);
+          c0 = 0;
+          c1 = 1;
+        } else {  // nothing follows: repeat the last tile (valid memory, never consumed)
+          c0 = c1 = ktiles - 1;
+        }
+      }
+      iteration(c0, I0{});
+      iteration(c1, I1{});
+    }
+  };
+
+  set_sources(cur);
+  copy_tile(0, 0);
+  copy_tile(1, 1);
+  // tile 0 must be complete, tile 1 may still be on its way
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kACopies + kBCopies));
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+
+  for (;;) {
+    local += wgs_per_xcd;
+    nxt = locate(local);
+    const int tile_rows = min(cur.row_end - cur.row_begin, BM);
+    const int live_blocks = (tile_rows + 31) / 32;
+    const int live = (live_blocks - wm + 1) / 2;
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    if (live >= MB) {
+      k_loop(std::integral_constant<int, MB>{});
+    } else if (MB > 1 && live == MB - 1) {
+      k_loop(std::integral_constant<int, (MB > 1 ? MB - 1 : 0)>{});
+    } else if (MB > 2 && live == MB - 2) {
+      k_loop(std::integral_constant<int, (MB > 2 ? MB - 2 : 0)>{});
+    } else if (live >= 1) {
+      k_loop(std::integral_constant<int, (MB > 3 ? MB - 3 : 1)>{});
+    } else {
+      k_loop(std::integral_constant<int, 0>{});
+    }
+
+    // Epilogue of `cur`.  acc[i][j][4g+e]: output row 32*(wm+2i) + fm, output column
+    // wn*32*NB + 32j + 8g + 4fq + e.  For a pair of column groups (g, g+1) the two lanes of a row
+    // (fq = 0, 1) exchange halves: v_permlane32_swap trades the upper 32 lanes of its first
+    // operand for the lower 32 lanes of its second, after which lane fq holds the 8 consecutive
+    // columns of group g+fq.
+    const int m_w = 32 * wm + fm;
+    if constexpr (SWIGLU) {
+      const int col_w = cur.n_tile * BNO + wn * 32;
+#pragma unroll
+      for (int i = 0; i < MB; ++i) {
+        const int m = m_w + 64 * i;
+        if (i < live && col_w < n_out) {  // wave uniform
+          const bool row_ok = m < tile_rows;
+          f16* yrow = y + (int64_t)(cur.row_begin + m) * n_out + col_w + 8 * fq;
+#pragma unroll
+          for (int gp = 0; gp < 2; ++gp) {
+            f16x4 p0, p1;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float g = acc[i][0][8 * gp + e];
+              const float u = acc[i][1][8 * gp + e];
+              const float ex = __builtin_amdgcn_exp2f(-1.4426950408889634f * g);
+              const f16 o = (f16)(g * u * __builtin_amdgcn_rcpf(1.0f + ex));
+              if (e < 4) p0[e] = o; else p1[e - 4] = o;
+            }
+            const u32x2 d0 = __builtin_bit_cast(u32x2, p0);
+            const u32x2 d1 = __builtin_bit_cast(u32x2, p1);
+            const auto lo = __builtin_amdgcn_permlane32_swap(d0[0], d1[0], false, false);
+            const auto hi = __builtin_amdgcn_permlane32_swap(d0[1], d1[1], false, false);
+            u32x4 out;
+            out[0] = lo[0];
+            out[1] = hi[0];
+            out[2] = lo[1];
+            out[3] = hi[1];
+            if (row_ok) st128(yrow + 16 * gp, __builtin_bit_cast(f16x8, out));
+          }
+        }
+      }
+    } else {
+    const int col_w = cur.n_tile * BN + wn * 32 * NB;
+#pragma unroll
+    for (int i = 0; i < MB; ++i) {
+      const int m = m_w + 64 * i;
+      if (i < live) {  // wave uniform: both lanes of every pair take part in the exchange
+        const bool row_ok = m < tile_rows;
+        f16* yrow = y + (int64_t)(cur.row_begin + m) * n + col_w + 8 * fq;
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+          if (col_w + 32 * j < n) {
+#pragma unroll
+            for (int gp = 0; gp < 2; ++gp) {
+              f16x4 p0, p1;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                p0[e] = (f16)acc[i][j][8 * gp + e];
+                p1[e] = (f16)acc[i][j][8 * gp + 4 + e];
+              }
+              const u32x2 d0 = __builtin_bit_cast(u32x2, p0);
+              const u32x2 d1 = __builtin_bit_cast(u32x2, p1);
+              const auto lo = __builtin_amdgcn_permlane32_swap(d0[0], d1[0], false, false);
+              const auto hi = __builtin_amdgcn_permlane32_swap(d0[1], d1[1], false, false);
+              u32x4 out;
+              out[0] = lo[0];
+              out[1] = hi[0];
+              out[2] = lo[1];
+              out[3] = hi[1];
+              if (row_ok) st128(yrow + 32 * j + 16 * gp, __builtin_bit_cast(f16x8, out));
+            }
+          }
+        }
+      }
+    }
+    }
+    if (!nxt.valid) break;
+    cur = nxt;
+  }
+  // the repeated last-tile copies must have landed before the LDS is released
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+}
+
+template <int MB, int NB, int WN, bool SWIGLU, bool GATHER = false>
+static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* group_list, f16* y,
+                                 int64_t rows, int k, int num_experts, int n, hipStream_t stream,
+                                 const int32_t* row_idx = nullptr, int idx_div = 1, int64_t x_rows = 1) {
+  constexpr int BM = 64 * MB;
+  constexpr int BN = 32 * NB * WN;
+  constexpr int kWaves = 2 * WN;
+  constexpr int kLds = 2 * (BM + BN) * kBK * (int)sizeof(f16) + kWaves * kWave * 8 * (int)sizeof(int);
+  static_assert(kLds <= 160 * 1024, "LDS budget");
+  static int cus[64] = {0};  // per device; benign race: every writer stores the same value
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return record_launch_status(e);
+  if (dev < 0 || dev >= 64) return AOPS_ERR_INVALID_ARGUMENT;
+  if (cus[dev] == 0) {
+    int v = 0;
+    e = hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return record_launch_status(e);
+    cus[dev] = v > 0 ? v : 8;
+  }
+  constexpr int BNO = SWIGLU ? BN / 2 : BN;
+  const int64_t n_out = SWIGLU ? n / 2 : n;
+  const int64_t n_tiles = (n_out + BNO - 1) / BNO;
+  const int64_t max_work = ((rows + BM - 1) / BM + num_experts) * n_tiles;
+  int64_t grid = cus[dev] < max_work ? cus[dev] : max_work;
+  grid = grid / kXcds * kXcds;
+  if (grid < kXcds) grid = kXcds;
+  auto kernel = grouped_matmul_persistent_kernel<MB, NB, WN, SWIGLU, GATHER>;
+  static bool attr_set = false;  // benign race: the call is idempotent
+  if (!attr_set) {
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return record_launch_status(e);
+    attr_set = true;
+  }
+  kernel<<<(unsigned)grid, 2 * WN * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts,
+                                                          n, row_idx, idx_div, (uint32_t)x_rows);
+  return record_launch_status(hipGetLastError());
+}
+
+int gmm_launch_persistent(bool swiglu, const f16* x, const f16* w, const int64_t* group_list, f16* y,
+                          int64_t rows, int k, int num_experts, int n, hipStream_t stream,
+                          const int32_t* row_idx, int idx_div, int64_t x_rows) {
+  if (row_idx)  // only the fused gate_up form gathers
+    return gmm_persistent_launch<5, 2, 4, true, true>(x, w, group_list, y, rows, k, num_experts, n, stream,
+                                                      row_idx, idx_div, x_rows);
+  if (swiglu) return gmm_persistent_launch<5, 2, 4, true>(x, w, group_list, y, rows, k, num_experts, n, stream);
+  return gmm_persistent_launch<5, 2, 4, false>(x, w, group_list, y, rows, k, num_experts, n, stream);
+}
+
+}  // namespace aops

@@ -1,0 +1,540 @@
+// Grouped matmul, one workgroup per work item: the register-staged kernel (four waves) and the
+// kernel that copies its operand tiles HBM -> LDS directly.
+#include "gmm_common.h"
+
+namespace aops {
+
+// Workgroup tile BM x BN = (64*MB) x (64*NB), four waves arranged 2 x 2.  Wave (wm, wn) owns
+// the 32-row blocks wm, wm+2, wm+4, ... (interleaved, so that a group that fills only part of
+// the tile still splits evenly between the two wave rows) and the 32*NB columns starting at
+// wn*32*NB; its MB x NB accumulators of v_mfma_f32_32x32x16_f16 stay in registers for the
+// whole k loop.  The products are formed as W.x^T (weight fragment as the first operand): a lane
+// then holds 4 consecutive output columns of one output row, which the epilogue packs to
+// 8 bytes, transposes through LDS and writes with 128-bit row-contiguous stores.
+//
+// Software pipeline per k tile (kBK = 64):
+//   global -> registers, D tiles ahead (the loads of tile kt+1+D are issued in iteration kt),
+//   registers -> LDS stage (kt+1)&1 during iteration kt, one barrier per k tile,
+//   LDS -> MFMA fragments one 16-wide k step ahead of the matrix cores.
+template <int MB, int NB, int D>
+__global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
+    const f16* __restrict__ x, const f16* __restrict__ w, const int64_t* __restrict__ group_list,
+    f16* __restrict__ y, int64_t rows, int k, int num_experts, int n) {
+  constexpr int BM = 64 * MB;
+  constexpr int BN = 64 * NB;
+  constexpr int kThreads = 4 * kWave;
+  constexpr int kAChunks = BM * (kBK / 8) / kThreads;  // 16-byte chunks per thread and tile
+  constexpr int kBChunks = BN * (kBK / 8) / kThreads;
+  constexpr int kRowsPerPass = kThreads / 8;           // tile rows covered by one chunk per thread
+  constexpr int kSteps = kBK / 16;
+  static_assert(D == 1 || D == 2, "prefetch distance");
+  static_assert(kRowsPerPass % 16 == 0, "swizzle must be invariant under the row stride");
+
+  extern __shared__ __attribute__((aligned(16))) f16 smem[];
+  f16* sa = smem;                 // [2][BM * kBK]
+  f16* sb = smem + 2 * BM * kBK;  // [2][BN * kBK]
+
+  const int n_tiles = (n + BN - 1) / BN;
+  const GmmWork work =
+      gmm_find_work<BM>(group_list, num_experts, rows, n_tiles, blockIdx.x, gridDim.x);
+  if (!work.valid) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave >> 1;
+  const int wn = wave & 1;
+  const int tile_rows = min(work.row_end - work.row_begin, BM);
+  // 32-row blocks of this wave that hold at least one real row (wave uniform, 0..MB)
+  const int live_blocks = (tile_rows + 31) / 32;
+  const int live = (live_blocks - wm + 1) / 2;
+
+  // Global -> register staging: thread handles chunk (row = tid/8 + kRowsPerPass*i, kc = tid%8).
+  // Sources are a uniform 64-bit tile base plus a 32-bit per-lane offset; LDS destinations are
+  // one per-lane offset plus compile-time strides.
+  const int ld_row = tid >> 3;
+  const int ld_kc = tid & 7;
+  const f16* a_base = x + (int64_t)work.row_begin * k;
+  const f16* b_base = w + ((int64_t)work.expert * n + (int64_t)work.n_tile * BN) * k;
+  uint32_t a_off[kAChunks], b_off[kBChunks];
+  const int n_left = n - work.n_tile * BN;  // rows of w available to this tile (>= 64)
+#pragma unroll
+  for (int i = 0; i < kAChunks; ++i) {
+    int ar = ld_row + kRowsPerPass * i;
+    if (ar > tile_rows - 1) ar = tile_rows - 1;  // rows past the group: duplicates, never stored
+    a_off[i] = (uint32_t)ar * (uint32_t)k + ld_kc * 8;
+  }
+#pragma unroll
+  for (int i = 0; i < kBChunks; ++i) {
+    int br = ld_row + kRowsPerPass * i;
+    if (br > n_left - 1) br = n_left - 1;  // n is a multiple of 64, not necessarily of BN
+    b_off[i] = (uint32_t)br * (uint32_t)k + ld_kc * 8;
+  }
+  const int st_dst = lds_off(ld_row, ld_kc);
+
+  f32x16 acc[MB][NB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  f16x8 ra[D][kAChunks], rb[D][kBChunks];  // D tiles in flight
+  const int ktiles = k / kBK;
+
+  auto load_tile = [&](int slot, int kt) {
+#pragma unroll
+    for (int i = 0; i < kAChunks; ++i) ra[slot][i] = ld128(a_base + kt * kBK + a_off[i]);
+#pragma unroll
+    for (int i = 0; i < kBChunks; ++i) rb[slot][i] = ld128_stream(b_base + kt * kBK + b_off[i]);
+  };
+  auto store_tile = [&](int slot, int stage) {
+    f16* da = sa + stage * BM * kBK;
+    f16* db = sb + stage * BN * kBK;
+#pragma unroll
+    for (int i = 0; i < kAChunks; ++i)
+      *reinterpret_cast<f16x8*>(&da[st_dst + i * kRowsPerPass * kBK]) = ra[slot][i];
+#pragma unroll
+    for (int i = 0; i < kBChunks; ++i)
+      *reinterpret_cast<f16x8*>(&db[st_dst + i * kRowsPerPass * kBK]) = rb[slot][i];
+  };
+
+  const int fm = lane & 31;  // fragment row inside a 32-row block
+  const int fq = lane >> 5;  // which half of a 16-wide k step
+  // Fragment reads: block offsets are compile-time strides on top of one per-lane offset per k
+  // step (the swizzle depends on fm and on the chunk only).
+  int frag_off[kSteps];
+#pragma unroll
+  for (int st = 0; st < kSteps; ++st) frag_off[st] = lds_off(fm, st * 2 + fq);
+  const f16* sa_w = sa + wm * 32 * kBK;
+  const f16* sb_w = sb + wn * 32 * NB * kBK;
+
+  // The k loop for LIVE live row blocks.  Iteration kt works on tile kt in LDS stage kt&1; the
+  // register slot (kt+1)%D holds tile kt+1.  Per iteration, four k steps of 16:
+  //   steps 0..2: MFMAs of the step | fragment reads of the next step (same stage) | a third of
+  //               the staging: LDS writes of tile kt+1 into the other stage, each followed by
+  //               the global load of tile kt+1+D into the register it just freed;
+  //   barrier   : every wave has read all its fragments of tile kt and written its part of
+  //               tile kt+1;
+  //   step 3    : MFMAs of the step | fragment reads of step 0 of tile kt+1.
+  // So the matrix cores never wait for an LDS round trip at a tile boundary, and there is one
+  // barrier per k tile.  Past the end of the k loop the same code runs on the last tile again
+  // (valid memory, results never consumed) instead of branching.
+  auto k_loop = [&](auto live_c) {
+    constexpr int LIVE = decltype(live_c)::value;
+    constexpr int kStageSteps = kSteps - 1;  // steps that carry staging traffic
+    constexpr int kAPer = (kAChunks + kStageSteps - 1) / kStageSteps;
+    constexpr int kBPer = (kBChunks + kStageSteps - 1) / kStageSteps;
+    f16x8 fa[2][LIVE > 0 ? LIVE : 1], fb[2][NB];
+    auto load_frags = [&](int buf, int st, int stage) {
+      const f16* ca = sa_w + stage * BM * kBK;
+      const f16* cb = sb_w + stage * BN * kBK;
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        fb[buf][j] = *reinterpret_cast<const f16x8*>(&cb[frag_off[st] + j * 32 * kBK]);
+#pragma unroll
+      for (int i = 0; i < LIVE; ++i)
+        fa[buf][i] = *reinterpret_cast<const f16x8*>(&ca[frag_off[st] + i * 64 * kBK]);
+    };
+    auto step = [&](int kload, auto slot_c, auto stage_c, auto st_c) {
+      constexpr int SLOT = decltype(slot_c)::value;
+      constexpr int STAGE = decltype(stage_c)::value;
+      constexpr int ST = decltype(st_c)::value;
+      constexpr int a_lo = ST * kAPer < kAChunks ? ST * kAPer : kAChunks;
+      constexpr int a_hi = (ST + 1) * kAPer < kAChunks ? (ST + 1) * kAPer : kAChunks;
+      constexpr int b_lo = ST * kBPer < kBChunks ? ST * kBPer : kBChunks;
+      constexpr int b_hi = (ST + 1) * kBPer < kBChunks ? (ST + 1) * kBPer : kBChunks;
+      constexpr int n_stage = ST < kStageSteps ? (a_hi - a_lo) + (b_hi - b_lo) : 0;
+      if (ST + 1 < kSteps) {
+        load_frags((ST + 1) & 1, ST + 1, STAGE);
+        f16* da = sa + (STAGE ^ 1) * BM * kBK;
+        f16* db = sb + (STAGE ^ 1) * BN * kBK;
+#pragma unroll
+        for (int i = a_lo; i < a_hi; ++i) {
+          *reinterpret_cast<f16x8*>(&da[st_dst + i * kRowsPerPass * kBK]) = ra[SLOT][i];
+          ra[SLOT][i] = ld128(a_base + kload + a_off[i]);
+        }
+#pragma unroll
+        for (int i = b_lo; i < b_hi; ++i) {
+          *reinterpret_cast<f16x8*>(&db[st_dst + i * kRowsPerPass * kBK]) = rb[SLOT][i];
+          rb[SLOT][i] = ld128_stream(b_base + kload + b_off[i]);
+        }
+      } else {
+        load_frags(0, 0, STAGE ^ 1);  // first fragments of the next tile
+      }
+#pragma unroll
+      for (int i = 0; i < LIVE; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ST & 1][j], fa[ST & 1][i],
+                                                             acc[i][j], 0, 0, 0);
+      MfmaInterleave<0, LIVE * NB, LIVE + NB, n_stage, n_stage>::run();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto iteration = [&](int kt, auto slot_c, auto stage_c) {
+      const int kload = min(kt + 1 + D, ktiles - 1) * kBK;
+      step(kload, slot_c, stage_c, std::integral_constant<int, 0>{});
+      step(kload, slot_c, stage_c, std::integral_constant<int, 1>{});
+      step(kload, slot_c, stage_c, std::integral_constant<int, 2>{});
+      __syncthreads();
+      step(kload, slot_c, stage_c, std::integral_constant<int, 3>{});
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    using SlotEven = std::integral_constant<int, 1 % D>;  // slot of tile kt+1 for even kt
+    using SlotOdd = std::integral_constant<int, 2 % D>;   // ... for odd kt
+    __syncthreads();  // tile 0 is in stage 0
+    load_frags(0, 0, 0);
+    int kt = 0;
+    for (; kt + 1 < ktiles; kt += 2) {
+      iteration(kt, SlotEven{}, I0{});
+      iteration(kt + 1, SlotOdd{}, I1{});
+    }
+    if (kt < ktiles) iteration(kt, SlotEven{}, I0{});
+  };
+
+  // tile t travels in register slot t % D and is consumed from LDS stage t & 1
+  load_tile(0, 0);
+  store_tile(0, 0);
+#pragma unroll
+  for (int t = 1; t <= D; ++t) load_tile(t % D, min(t, ktiles - 1));
+  // One branch-free instantiation of the k loop per number of live row blocks.
+  if (live >= MB) {
+    k_loop(std::integral_constant<int, MB>{});
+  } else if (MB > 1 && live == MB - 1) {
+    k_loop(std::integral_constant<int, (MB > 1 ? MB - 1 : 0)>{});
+  } else if (MB > 2 && live == MB - 2) {
+    k_loop(std::integral_constant<int, (MB > 2 ? MB - 2 : 0)>{});
+  } else if (live >= 1) {  // short groups: rarely worth a dedicated copy, use the next larger one
+    if (MB > 3 && live <= MB - 3) k_loop(std::integral_constant<int, (MB > 3 ? MB - 3 : 0)>{});
+  } else {
+    k_loop(std::integral_constant<int, 0>{});
+  }
+
+  // Epilogue.  acc[i][j][r]: output row 32*(wm+2i) + lane%32, output columns
+  // wn*32*NB + 32j + 8*(r/4) + 4*(lane/32) + r%4.  The C tile goes to LDS as [BM][BN] halfs in
+  // 8-byte pieces, piece c of row m at position c ^ ((m & kSwz) << 1) (write conflicts at most
+  // 2-way, 16-byte reads stay contiguous), and leaves as 128-bit row-contiguous global stores.
+  __syncthreads();  // all waves are done with the operand stages
+  f16* sc = smem;
+  constexpr int kSwz = (BN / 8 < 16 ? BN / 8 : 16) - 1;  // swizzle stays inside the row
+#pragma unroll
+  for (int i = 0; i < MB; ++i) {
+    const int m = 32 * (wm + 2 * i) + fm;
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f16x4 v;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (f16)acc[i][j][4 * g + e];
+        const int piece = (wn * 32 * NB + 32 * j + 8 * g + 4 * fq) >> 2;
+        *reinterpret_cast<f16x4*>(&sc[m * BN + ((piece ^ ((m & kSwz) << 1)) << 2)]) = v;
+      }
+    }
+  }
+  __syncthreads();
+  constexpr int kChunksPerRow = BN / 8;              // 16-byte chunks per tile row
+  constexpr int kRowsPerStorePass = kThreads / kChunksPerRow;
+  const int c16 = tid % kChunksPerRow;
+  const int col = work.n_tile * BN + c16 * 8;
+  if (col < n) {
+    for (int m = tid / kChunksPerRow; m < tile_rows; m += kRowsPerStorePass) {
+      const f16x8 v = *reinterpret_cast<const f16x8*>(&sc[m * BN + ((c16 ^ (m & kSwz)) << 3)]);
+      st128(y + (int64_t)(work.row_begin + m) * n + col, v);
+    }
+  }
+}
+
+// Same tiling and MFMA work as grouped_matmul_kernel, but both operand tiles travel HBM -> LDS
+// directly (global_load_lds_dwordx4: 64 lanes deposit 64 consecutive 16-byte chunks), so the k
+// loop holds no staging registers and issues no LDS writes.  Because a lane cannot choose where
+// its chunk lands, the swizzle is applied on the source side: the lane that owns physical chunk
+// (row pr, position pc) fetches logical chunk (pr ^ ((pr>>3)&1), pc ^ (row & 7)).
+// Two LDS stages.  Per tile kt (stage kt&1), four k steps of 16:
+//   steps 0..2: MFMAs | fragment reads of the next step
+//   then      : wait for this wave's copies of tile kt+1, barrier (tile kt+1 complete for
+//               everyone, nobody reads stage kt&1 any more)
+//   step 3    : MFMAs | fragment reads of step 0 of tile kt+1 | copies of tile kt+2 into stage kt&1
+template <int MB, int NB, int WN>
+__global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
+    const f16* __restrict__ x, const f16* __restrict__ w, const int64_t* __restrict__ group_list,
+    f16* __restrict__ y, int64_t rows, int k, int num_experts, int n) {
+  constexpr int kWaves = 2 * WN;  // 2 wave rows x WN wave columns
+  constexpr int BM = 64 * MB;
+  constexpr int BN = 32 * NB * WN;
+  constexpr int kThreads = kWaves * kWave;
+  constexpr int kSteps = kBK / 16;
+  constexpr int kACopies = BM / 8 / kWaves;  // copy instructions per wave and tile (8 rows each)
+  constexpr int kBCopies = BN / 8 / kWaves;
+  static_assert(BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0, "tile rows per copy");
+
+  extern __shared__ __attribute__((aligned(16))) f16 smem[];
+  f16* sa = smem;                 // [2][BM * kBK]
+  f16* sb = smem + 2 * BM * kBK;  // [2][BN * kBK]
+
+  const int n_tiles = (n + BN - 1) / BN;
+  const GmmWork work =
+      gmm_find_work<BM>(group_list, num_experts, rows, n_tiles, blockIdx.x, gridDim.x);
+  if (!work.valid) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave / WN;
+  const int wn = wave % WN;
+  const int tile_rows = min(work.row_end - work.row_begin, BM);
+  const int live_blocks = (tile_rows + 31) / 32;
+  const int live = (live_blocks - wm + 1) / 2;
+
+  // Copy sources.  Copy i of this wave fills physical rows (kWaves*i + wave)*8 .. +7 of a stage.
+  const f16* a_base = x + (int64_t)work.row_begin * k;
+  const f16* b_base = w + ((int64_t)work.expert * n + (int64_t)work.n_tile * BN) * k;
+  const int n_left = n - work.n_tile * BN;                      // rows of w available (>= 64)
+  const int64_t x_left = rows - work.row_begin;                 // rows of x available (>= 1)
+  uint32_t a_off[kACopies], b_off[kBCopies];
+  {
+    const int pr_lo = lane >> 3;  // physical row inside the 8-row group
+    const int pc = lane & 7;      // physical chunk position
+#pragma unroll
+    for (int i = 0; i < kACopies; ++i) {
+      const int pr = (kWaves * i + wave) * 8 + pr_lo;
+      int r = pr ^ ((pr >> 3) & 1);
+      const int c = pc ^ (r & 7);
+      // rows past the group read whatever follows in x (only dead output rows depend on them);
+      // rows past the end of x are clamped
+      if (r > x_left - 1) r = (int)(x_left - 1);
+      a_off[i] = (uint32_t)r * (uint32_t)k + c * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < kBCopies; ++i) {
+      const int pr = (kWaves * i + wave) * 8 + pr_lo;
+      int r = pr ^ ((pr >> 3) & 1);
+      const int c = pc ^ (r & 7);
+      if (r > n_left - 1) r = n_left - 1;
+      b_off[i] = (uint32_t)r * (uint32_t)k + c * 8;
+    }
+  }
+  const int ktiles = k / kBK;
+  auto copy_tile = [&](int kt, int stage) {
+    const int ko = min(kt, ktiles - 1) * kBK;
+    f16* da = sa + stage * BM * kBK + wave * 512;
+    f16* db = sb + stage * BN * kBK + wave * 512;
+#pragma unroll
+    for (int i = 0; i < kACopies; ++i)
+      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(a_base + ko + a_off[i]),
+                                       AOPS_LDS_PTR(da + i * kWaves * 512), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < kBCopies; ++i)
+      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(b_base + ko + b_off[i]),
+                                       AOPS_LDS_PTR(db + i * kWaves * 512), 16, 0, 0);
+  };
+
+  f32x16 acc[MB][NB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int fm = lane & 31;
+  const int fq = lane >> 5;
+  int frag_off[kSteps];
+#pragma unroll
+  for (int st = 0; st < kSteps; ++st) frag_off[st] = lds_off(fm, st * 2 + fq);
+  const f16* sa_w = sa + wm * 32 * kBK;
+  const f16* sb_w = sb + wn * 32 * NB * kBK;
+
+  auto k_loop = [&](auto live_c) {
+    constexpr int LIVE = decltype(live_c)::value;
+    f16x8 fa[2][LIVE > 0 ? LIVE : 1], fb[2][NB];
+    auto load_frags = [&](int buf, int st, int stage) {
+      const f16* ca = sa_w + stage * BM * kBK;
+      const f16* cb = sb_w + stage * BN * kBK;
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        fb[buf][j] = *reinterpret_cast<const f16x8*>(&cb[frag_off[st] + j * 32 * kBK]);
+#pragma unroll
+      for (int i = 0; i < LIVE; ++i)
+        fa[buf][i] = *reinterpret_cast<const f16x8*>(&ca[frag_off[st] + i * 64 * kBK]);
+    };
+    auto step = [&](int kt, auto stage_c, auto st_c) {
+      constexpr int STAGE = decltype(stage_c)::value;
+      constexpr int ST = decltype(st_c)::value;
+      if (ST + 1 < kSteps) {
+        load_frags((ST + 1) & 1, ST + 1, STAGE);
+      } else {
+        load_frags(0, 0, STAGE ^ 1);  // first fragments of the next tile
+        copy_tile(kt + 2, STAGE);     // this stage is free: everyone is past the barrier
+      }
+#pragma unroll
+      for (int i = 0; i < LIVE; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ST & 1][j], fa[ST & 1][i],
+                                                             acc[i][j], 0, 0, 0);
+      MfmaInterleave<0, LIVE * NB, LIVE + NB, 0,
+                     (ST + 1 < kSteps) ? 0 : kACopies + kBCopies>::run();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto iteration = [&](int kt, auto stage_c) {
+      step(kt, stage_c, std::integral_constant<int, 0>{});
+      step(kt, stage_c, std::integral_constant<int, 1>{});
+      step(kt, stage_c, std::integral_constant<int, 2>{});
+      // own copies of tile kt+1 and all own fragment reads of tile kt are complete ...
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();  // ... and so are everybody else's
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+      step(kt, stage_c, std::integral_constant<int, 3>{});
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    // tile 0 must be complete, tile 1 may still be on its way
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kACopies + kBCopies));
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    load_frags(0, 0, 0);
+    int kt = 0;
+    for (; kt + 1 < ktiles; kt += 2) {
+      iteration(kt, I0{});
+      iteration(kt + 1, I1{});
+    }
+    if (kt < ktiles) iteration(kt, I0{});
+  };
+
+  copy_tile(0, 0);
+  copy_tile(1, 1);
+  if (live >= MB) {
+    k_loop(std::integral_constant<int, MB>{});
+  } else if (MB > 1 && live == MB - 1) {
+    k_loop(std::integral_constant<int, (MB > 1 ? MB - 1 : 0)>{});
+  } else if (MB > 2 && live == MB - 2) {
+    k_loop(std::integral_constant<int, (MB > 2 ? MB - 2 : 0)>{});
+  } else if (live >= 1) {
+    if (MB > 3 && live <= MB - 3) k_loop(std::integral_constant<int, (MB > 3 ? MB - 3 : 0)>{});
+  } else {
+    k_loop(std::integral_constant<int, 0>{});
+  }
+
+  // Epilogue: as in grouped_matmul_kernel, one pass per pair of wave columns (BM x 64*NB halfs fit
+  // the stages).  The last copies (a repeat of the last tile) must have landed before the stages
+  // are reused for the output tile.
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+  __syncthreads();
+  f16* sc = smem;
+  constexpr int kPassCols = 64 * NB;  // columns of two wave columns
+  constexpr int kSwz = (kPassCols / 8 < 16 ? kPassCols / 8 : 16) - 1;
+  constexpr int kChunksPerRow = kPassCols / 8;
+  constexpr int kRowsPerStorePass = kThreads / kChunksPerRow;
+#pragma unroll
+  for (int pass = 0; pass < WN / 2; ++pass) {
+    if (wn / 2 == pass) {
+#pragma unroll
+      for (int i = 0; i < MB; ++i) {
+        const int m = 32 * (wm + 2 * i) + fm;
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            f16x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = (f16)acc[i][j][4 * g + e];
+            const int piece = ((wn & 1) * 32 * NB + 32 * j + 8 * g + 4 * fq) >> 2;
+            *reinterpret_cast<f16x4*>(&sc[m * kPassCols + ((piece ^ ((m & kSwz) << 1)) << 2)]) = v;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    const int c16 = tid % kChunksPerRow;
+    const int col = work.n_tile * BN + pass * kPassCols + c16 * 8;
+    if (col < n) {
+      for (int m = tid / kChunksPerRow; m < tile_rows; m += kRowsPerStorePass) {
+        const f16x8 v =
+            *reinterpret_cast<const f16x8*>(&sc[m * kPassCols + ((c16 ^ (m & kSwz)) << 3)]);
+        st128(y + (int64_t)(work.row_begin + m) * n + col, v);
+      }
+    }
+    if (pass + 1 < WN / 2) __syncthreads();
+  }
+}
+
+template <int MB, int NB, int WN>
+static int gmm_dma_launch(const f16* x, const f16* w, const int64_t* group_list, f16* y,
+                          int64_t rows, int k, int num_experts, int n, hipStream_t stream) {
+  constexpr int BM = 64 * MB;
+  constexpr int BN = 32 * NB * WN;
+  constexpr int kStageBytes = 2 * (BM + BN) * kBK * (int)sizeof(f16);
+  constexpr int kTileBytes = BM * 64 * NB * (int)sizeof(f16);
+  constexpr int kLds = kStageBytes > kTileBytes ? kStageBytes : kTileBytes;
+  static_assert(kLds <= 160 * 1024, "LDS budget");
+  const int64_t n_tiles = (n + BN - 1) / BN;
+  const int64_t max_m_tiles = (rows + BM - 1) / BM + num_experts;
+  int64_t grid = max_m_tiles * n_tiles;
+  grid = (grid + kXcds - 1) / kXcds * kXcds;
+  if (grid > 0x7fffffff) return AOPS_ERR_INVALID_ARGUMENT;
+  auto kernel = grouped_matmul_dma_kernel<MB, NB, WN>;
+  static bool attr_set = false;  // benign race: the call is idempotent
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return record_launch_status(e);
+    attr_set = true;
+  }
+  kernel<<<(unsigned)grid, 2 * WN * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts,
+                                                          n);
+  return record_launch_status(hipGetLastError());
+}
+
+template <int MB, int NB, int D>
+static int gmm_launch(const f16* x, const f16* w, const int64_t* group_list, f16* y, int64_t rows,
+                      int k, int num_experts, int n, hipStream_t stream) {
+  constexpr int BM = 64 * MB;
+  constexpr int BN = 64 * NB;
+  constexpr int kStageBytes = 2 * (BM + BN) * kBK * (int)sizeof(f16);
+  constexpr int kTileBytes = BM * BN * (int)sizeof(f16);
+  constexpr int kLds = kStageBytes > kTileBytes ? kStageBytes : kTileBytes;
+  static_assert(kLds <= 160 * 1024, "LDS budget");
+  const int64_t n_tiles = (n + BN - 1) / BN;
+  const int64_t max_m_tiles = (rows + BM - 1) / BM + num_experts;
+  int64_t grid = max_m_tiles * n_tiles;
+  grid = (grid + kXcds - 1) / kXcds * kXcds;
+  if (grid > 0x7fffffff) return AOPS_ERR_INVALID_ARGUMENT;
+  auto kernel = grouped_matmul_kernel<MB, NB, D>;
+  static bool attr_set = false;  // benign race: the call is idempotent
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) return record_launch_status(e);
+    attr_set = true;
+  }
+  kernel<<<(unsigned)grid, 4 * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts, n);
+  return record_launch_status(hipGetLastError());
+}
+
+int gmm_launch_tiles(int variant, const f16* x, const f16* w, const int64_t* group_list, f16* y,
+                     int64_t rows, int k, int num_experts, int n, hipStream_t stream) {
+  switch (variant) {
+    case 1:  // 320 x 256 tiles, eight waves, operands copied HBM -> LDS directly
+      return gmm_dma_launch<5, 2, 4>(x, w, group_list, y, rows, k, num_experts, n, stream);
+    case 7:  // 256 x 128 tiles, four waves, operands copied HBM -> LDS directly
+      return gmm_dma_launch<4, 2, 2>(x, w, group_list, y, rows, k, num_experts, n, stream);
+    case 8:  // 128 x 128 tiles, four waves, operands copied HBM -> LDS directly
+      return gmm_dma_launch<2, 2, 2>(x, w, group_list, y, rows, k, num_experts, n, stream);
+    case 2:  // 320 x 128 tiles
+      return gmm_launch<5, 2, 2>(x, w, group_list, y, rows, k, num_experts, n, stream);
+    case 3:  // 256 x 128 tiles
+      return gmm_launch<4, 2, 2>(x, w, group_list, y, rows, k, num_experts, n, stream);
+    case 4:  // 128 x 128 tiles
+      return gmm_launch<2, 2, 2>(x, w, group_list, y, rows, k, num_experts, n, stream);
+    default:  // 64 x 64 tiles
+      return gmm_launch<1, 1, 2>(x, w, group_list, y, rows, k, num_experts, n, stream);
+  }
+}
+
+}  // namespace aops
