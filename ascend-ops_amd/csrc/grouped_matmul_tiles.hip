@@ -288,47 +288,41 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
   const int live_blocks = (tile_rows + 31) / 32;
   const int live = (live_blocks - wm + 1) / 2;
 
-  // Copy sources.  Copy i of this wave fills physical rows (kWaves*i + wave)*8 .. +7 of a stage.
+  // Copy sources.  Copy i of this wave fills physical rows (kWaves*i + wave)*8 .. +7 of a stage,
+  // i.e. logical row 8*kWaves*i + lane_row (the row swizzle only swaps rows inside the 8-row group)
+  // and chunk lane_c: one per-lane offset plus a uniform stride per copy, clamped to the last valid
+  // row (tile rows past the end of the group - only dead output rows depend on them - and past
+  // the end of w repeat the last valid row).
   const f16* a_base = x + (int64_t)work.row_begin * k;
   const f16* b_base = w + ((int64_t)work.expert * n + (int64_t)work.n_tile * BN) * k;
-  const int n_left = n - work.n_tile * BN;                      // rows of w available (>= 64)
-  const int64_t x_left = rows - work.row_begin;                 // rows of x available (>= 1)
-  uint32_t a_off[kACopies], b_off[kBCopies];
-  {
-    const int pr_lo = lane >> 3;  // physical row inside the 8-row group
-    const int pc = lane & 7;      // physical chunk position
-#pragma unroll
-    for (int i = 0; i < kACopies; ++i) {
-      const int pr = (kWaves * i + wave) * 8 + pr_lo;
-      int r = pr ^ ((pr >> 3) & 1);
-      const int c = pc ^ (r & 7);
-      // rows past the group read whatever follows in x (only dead output rows depend on them);
-      // rows past the end of x are clamped
-      if (r > x_left - 1) r = (int)(x_left - 1);
-      a_off[i] = (uint32_t)r * (uint32_t)k + c * 8;
-    }
-#pragma unroll
-    for (int i = 0; i < kBCopies; ++i) {
-      const int pr = (kWaves * i + wave) * 8 + pr_lo;
-      int r = pr ^ ((pr >> 3) & 1);
-      const int c = pc ^ (r & 7);
-      if (r > n_left - 1) r = n_left - 1;
-      b_off[i] = (uint32_t)r * (uint32_t)k + c * 8;
-    }
-  }
+  const int n_left = min(n - work.n_tile * BN, BN);
+  const int lane_row = wave * 8 + ((lane >> 3) ^ (wave & 1));
+  const int lane_c = (lane & 7) ^ (lane_row & 7);
+  const uint32_t off0 = (uint32_t)lane_row * (uint32_t)k + lane_c * 8;
+  const uint32_t copy_stride = 8u * kWaves * (uint32_t)k;
+  const uint32_t a_last = (uint32_t)(tile_rows - 1) * (uint32_t)k + lane_c * 8;
+  const uint32_t b_last = (uint32_t)(n_left - 1) * (uint32_t)k + lane_c * 8;
   const int ktiles = k / kBK;
   auto copy_tile = [&](int kt, int stage) {
     const int ko = min(kt, ktiles - 1) * kBK;
     f16* da = sa + stage * BM * kBK + wave * 512;
     f16* db = sb + stage * BN * kBK + wave * 512;
+    // the empty asm makes the 64-bit source address of a copy be formed right before the copy
+    // instead of being kept in a register pair per copy across the k loop
 #pragma unroll
-    for (int i = 0; i < kACopies; ++i)
-      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(a_base + ko + a_off[i]),
+    for (int i = 0; i < kACopies; ++i) {
+      uint32_t o = min(off0 + i * copy_stride, a_last);
+      asm volatile("" : "+v"(o));
+      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(a_base + ko + o),
                                        AOPS_LDS_PTR(da + i * kWaves * 512), 16, 0, 0);
+    }
 #pragma unroll
-    for (int i = 0; i < kBCopies; ++i)
-      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(b_base + ko + b_off[i]),
+    for (int i = 0; i < kBCopies; ++i) {
+      uint32_t o = min(off0 + i * copy_stride, b_last);
+      asm volatile("" : "+v"(o));
+      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(b_base + ko + o),
                                        AOPS_LDS_PTR(db + i * kWaves * 512), 16, 0, 0);
+    }
   };
 
   f32x16 acc[MB][NB];
@@ -341,24 +335,27 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
 
   const int fm = lane & 31;
   const int fq = lane >> 5;
-  int frag_off[kSteps];
-#pragma unroll
-  for (int st = 0; st < kSteps; ++st) frag_off[st] = lds_off(fm, st * 2 + fq);
-  const f16* sa_w = sa + wm * 32 * kBK;
-  const f16* sb_w = sb + wn * 32 * NB * kBK;
+  // Fragment addresses: lds_off(fm, 2*st + fq) == lds_off(fm, fq) ^ (st << 4) (the k step only
+  // flips two chunk bits), so one per-lane offset per operand serves every k step.
+  const int fa_off0 = lds_off(fm, fq) + wm * 32 * kBK;
+  const int fb_off0 = lds_off(fm, fq) + wn * 32 * NB * kBK;
 
   auto k_loop = [&](auto live_c) {
     constexpr int LIVE = decltype(live_c)::value;
     f16x8 fa[2][LIVE > 0 ? LIVE : 1], fb[2][NB];
     auto load_frags = [&](int buf, int st, int stage) {
-      const f16* ca = sa_w + stage * BM * kBK;
-      const f16* cb = sb_w + stage * BN * kBK;
+      // the empty asm keeps the compiler from hoisting one address register per (stage, step)
+      // out of the k loop, which would push the accumulators into scratch
+      int fo_a = fa_off0, fo_b = fb_off0;
+      asm volatile("" : "+v"(fo_a), "+v"(fo_b));
+      const f16* ca = sa + stage * BM * kBK + (fo_a ^ (st << 4));
+      const f16* cb = sb + stage * BN * kBK + (fo_b ^ (st << 4));
 #pragma unroll
       for (int j = 0; j < NB; ++j)
-        fb[buf][j] = *reinterpret_cast<const f16x8*>(&cb[frag_off[st] + j * 32 * kBK]);
+        fb[buf][j] = *reinterpret_cast<const f16x8*>(&cb[j * 32 * kBK]);
 #pragma unroll
       for (int i = 0; i < LIVE; ++i)
-        fa[buf][i] = *reinterpret_cast<const f16x8*>(&ca[frag_off[st] + i * 64 * kBK]);
+        fa[buf][i] = *reinterpret_cast<const f16x8*>(&ca[i * 64 * kBK]);
     };
     auto step = [&](int kt, auto stage_c, auto st_c) {
       constexpr int STAGE = decltype(stage_c)::value;
