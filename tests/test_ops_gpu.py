@@ -438,6 +438,20 @@ def test_paged_attention(ops, dev, B, Hq, Hkv, P, lens):
     assert (o.float() - ref.float()).abs().max() < 2e-3
 
 
+def test_paged_attention_batch_larger_than_a_wave(ops, dev):
+    """More than 64 sequences: the longest-first ordering of the workgroups (one length per lane) is off and the
+    sequences are taken in index order; several chunks per sequence when the batch alone fills the chip."""
+    rnd = torch.Generator().manual_seed(12)
+    B = 150
+    lens = torch.randint(0, 600, (B,), generator=rnd).tolist()
+    lens[3] = 0
+    lens[77] = 2500
+    case = _paged_case(B, 8, 2, 128, 64, lens, seed=12)
+    o = _run_pa(ops, dev, case)
+    ref = R.paged_attention_ref(*case)
+    torch.testing.assert_close(o.float(), ref.float(), **TOL)
+
+
 @pytest.mark.parametrize(
     "B,Hq,Hkv,D,P,lens",
     [
