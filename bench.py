@@ -608,6 +608,8 @@ def main():
 
     import torch
 
+    import __graft_entry__ as entry_points
+    entry_points._build_if_absent()          # a fresh checkout holds no built library
     import ascend910a_extras.ops as ops      # the product; raises if libaops.so is missing
     import oracle.ops_ref as R               # checker + timed CPU baseline only
 
