@@ -84,9 +84,10 @@ def exported_symbols() -> list[str]:
     return sorted(_SIGNATURES)
 
 
-def _check(cond: bool, msg: str) -> None:
+def _check(cond: bool, msg) -> None:
+    """``msg`` is a string or a callable that builds one: messages are only formatted on failure."""
     if not cond:
-        raise RuntimeError(msg)
+        raise RuntimeError(msg() if callable(msg) else msg)
 
 
 def _status(op: str, code: int) -> None:
@@ -100,14 +101,23 @@ def _require_device(op: str, dtype_by_name: dict) -> None:
     """dtype and device checks (the reference hard-codes ACL_FLOAT16/ACL_INT32/ACL_INT64)."""
     device = None
     for name, (t, dtype) in dtype_by_name.items():
-        _check(t.dtype == dtype, f"{op}: {name} must be {dtype}, got {t.dtype}")
-        _check(t.is_cuda, f"{op}: {name} must be on the GPU device, got {t.device}")
+        if t.dtype != dtype:
+            raise RuntimeError(f"{op}: {name} must be {dtype}, got {t.dtype}")
+        if not t.is_cuda:
+            raise RuntimeError(f"{op}: {name} must be on the GPU device, got {t.device}")
         if device is None:
             device = t.device
-        _check(t.device == device, f"{op}: all tensors must be on the same device")
+        elif t.device != device:
+            raise RuntimeError(f"{op}: all tensors must be on the same device")
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _stream(device: torch.device) -> int:
+    """Raw handle of torch's current stream on ``device``."""
+    if _raw_stream is not None:
+        return _raw_stream(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -119,12 +129,12 @@ def rope(q, k, position_ids, cos_cache, sin_cache):
     """reference csrc/ffi/ops.cpp:13-108."""
     _check(
         q.dim() == 3 and k.dim() == 3 and position_ids.dim() == 1 and cos_cache.dim() == 2 and sin_cache.dim() == 2,
-        f"rope: input tensors must be 3D, 3D, 1D, 2D, and 2D, got {q.dim()}D, {k.dim()}D, "
+        lambda: f"rope: input tensors must be 3D, 3D, 1D, 2D, and 2D, got {q.dim()}D, {k.dim()}D, "
         f"{position_ids.dim()}D, {cos_cache.dim()}D, {sin_cache.dim()}D",
     )
     _check(
         position_ids.size(0) == q.size(0),
-        f"rope: position_ids must have the same batch size as q, got {position_ids.size(0)} and {q.size(0)}",
+        lambda: f"rope: position_ids must have the same batch size as q, got {position_ids.size(0)} and {q.size(0)}",
     )
     _check(
         q.is_contiguous() and k.is_contiguous() and position_ids.is_contiguous()
@@ -133,10 +143,10 @@ def rope(q, k, position_ids, cos_cache, sin_cache):
     )
     bs, num_heads, head_dim = q.shape
     _check(k.size(0) == bs and k.size(2) == head_dim, "rope: k must match q in batch size and head_dim")
-    _check(head_dim % 16 == 0, f"rope: head_dim must be a multiple of 16, got {head_dim}")
+    _check(head_dim % 16 == 0, lambda: f"rope: head_dim must be a multiple of 16, got {head_dim}")
     _check(
         cos_cache.size(1) == head_dim // 2 and sin_cache.shape == cos_cache.shape,
-        f"rope: cos_cache and sin_cache must be [max_position, head_dim/2], got {tuple(cos_cache.shape)} "
+        lambda: f"rope: cos_cache and sin_cache must be [max_position, head_dim/2], got {tuple(cos_cache.shape)} "
         f"and {tuple(sin_cache.shape)}",
     )
     _require_device(
@@ -158,10 +168,10 @@ def rope(q, k, position_ids, cos_cache, sin_cache):
 
 def swiglu(x):
     """reference csrc/ffi/ops.cpp:110-154."""
-    _check(x.dim() == 2, f"swiglu: input tensor must be 2D, got {x.dim()}D tensor")
+    _check(x.dim() == 2, lambda: f"swiglu: input tensor must be 2D, got {x.dim()}D tensor")
     _check(
         x.size(-1) >= 64 and x.size(-1) % 64 == 0,
-        f"swiglu: last dimension must be a multiple of 64, got {x.size(-1)}",
+        lambda: f"swiglu: last dimension must be a multiple of 64, got {x.size(-1)}",
     )
     _check(x.is_contiguous(), "swiglu: input tensor must be contiguous")
     _require_device("swiglu", {"x": (x, torch.float16)})
@@ -175,33 +185,33 @@ def _check_grouped_matmul(name, x, w, group_list):
     """Argument checks of reference csrc/ffi/ops.cpp:158-174 plus dtype, device and packing."""
     _check(
         x.dim() == 2 and w.dim() == 3 and group_list.dim() == 1,
-        f"{name}: input tensors must be 2D and group_list must be 1D",
+        lambda: f"{name}: input tensors must be 2D and group_list must be 1D",
     )
     dim = x.size(1)
     num_experts, inner_dim = w.size(0), w.size(2)
     _check(
         dim == w.size(1),
-        f"{name}: last dimension of x must match second dimension of w, got {dim} and {w.size(1)}",
+        lambda: f"{name}: last dimension of x must match second dimension of w, got {dim} and {w.size(1)}",
     )
     _check(
         x.is_contiguous() and group_list.is_contiguous(),
-        f"{name}: x and group_list must be contiguous tensors",
+        lambda: f"{name}: x and group_list must be contiguous tensors",
     )
     _check(
         w.stride(1) == 1 and w.stride(2) == dim,
-        f"{name}: w must be K-major order, got strides {tuple(w.stride())}",
+        lambda: f"{name}: w must be K-major order, got strides {tuple(w.stride())}",
     )
     _check(
         w.size(1) % 64 == 0 and w.size(2) % 64 == 0,
-        f"{name}: second and third dimensions of w must be multiples of 64, got {w.size(1)} and {w.size(2)}",
+        lambda: f"{name}: second and third dimensions of w must be multiples of 64, got {w.size(1)} and {w.size(2)}",
     )
     _check(
         num_experts <= 1 or w.stride(0) == dim * inner_dim,
-        f"{name}: experts of w must be densely packed, got strides {tuple(w.stride())}",
+        lambda: f"{name}: experts of w must be densely packed, got strides {tuple(w.stride())}",
     )
     _check(
         group_list.size(0) == num_experts,
-        f"{name}: group_list must have one entry per expert, got {group_list.size(0)} and {num_experts}",
+        lambda: f"{name}: group_list must have one entry per expert, got {group_list.size(0)} and {num_experts}",
     )
     _require_device(
         name,
@@ -227,12 +237,12 @@ def matmul(x, w):
     _check(x.dim() == 2 and w.dim() == 2, "matmul: input tensors must be 2D")
     _check(
         x.size(1) == w.size(1),
-        f"matmul: last dimension of x must match last dimension of w, got {x.size(1)} and {w.size(1)}",
+        lambda: f"matmul: last dimension of x must match last dimension of w, got {x.size(1)} and {w.size(1)}",
     )
     _check(x.is_contiguous() and w.is_contiguous(), "matmul: x and w must be contiguous tensors")
     m, k = x.shape
     n = w.size(0)
-    _check(k % 64 == 0 and n % 64 == 0, f"matmul: k and n must be multiples of 64, got k={k} and n={n}")
+    _check(k % 64 == 0 and n % 64 == 0, lambda: f"matmul: k and n must be multiples of 64, got k={k} and n={n}")
     _require_device("matmul", {"x": (x, torch.float16), "w": (w, torch.float16)})
     y = torch.empty((m, n), dtype=x.dtype, device=x.device)
     code = _lib.aops_matmul_nt_f16(_ptr(x), _ptr(w), _ptr(y), m, k, n, _stream(x.device))
@@ -265,17 +275,17 @@ def add_rms_norm(x, residual, weight, epsilon):
     )
     _check(
         x.size(1) == weight.size(0),
-        f"add_rms_norm: last dimension of x must match weight size, got {x.size(1)} and {weight.size(0)}",
+        lambda: f"add_rms_norm: last dimension of x must match weight size, got {x.size(1)} and {weight.size(0)}",
     )
     _check(
         x.size(0) == residual.size(0) and x.size(1) == residual.size(1),
-        f"add_rms_norm: x and residual must have the same shape, got {tuple(x.shape)} and {tuple(residual.shape)}",
+        lambda: f"add_rms_norm: x and residual must have the same shape, got {tuple(x.shape)} and {tuple(residual.shape)}",
     )
     _check(
         x.is_contiguous() and residual.is_contiguous() and weight.is_contiguous(),
         "add_rms_norm: all input tensors must be contiguous",
     )
-    _check(x.size(1) % 64 == 0, f"add_rms_norm: last dimension must be a multiple of 64, got {x.size(1)}")
+    _check(x.size(1) % 64 == 0, lambda: f"add_rms_norm: last dimension must be a multiple of 64, got {x.size(1)}")
     _require_device(
         "add_rms_norm",
         {"x": (x, torch.float16), "residual": (residual, torch.float16), "weight": (weight, torch.float16)},
@@ -312,11 +322,11 @@ def reshape_and_cache(key, value, key_cache, value_cache, slot_indices):
     # reference csrc/opdev/op_host/reshape_and_cache_ex.cpp:31-36
     _check(
         slot_indices.size(0) == num_tokens,
-        f"reshape_and_cache: slot_indices length must equal num_tokens, got {slot_indices.size(0)} and {num_tokens}",
+        lambda: f"reshape_and_cache: slot_indices length must equal num_tokens, got {slot_indices.size(0)} and {num_tokens}",
     )
     _check(
         chunk == 16 and nh16 * 16 == num_kv_heads * head_size,
-        f"reshape_and_cache: key_cache must be [num_blocks, num_kv_heads*head_size/16, block_size, 16], "
+        lambda: f"reshape_and_cache: key_cache must be [num_blocks, num_kv_heads*head_size/16, block_size, 16], "
         f"got {tuple(key_cache.shape)} for key {tuple(key.shape)}",
     )
     tensors = {
@@ -354,16 +364,16 @@ def paged_attention(q, key_cache, value_cache, block_tables, context_lens):
     )
     bs, num_heads, head_dim = q.shape
     num_blocks, nh16, block_size, chunk = key_cache.shape
-    _check(chunk == 16, f"paged_attention: last dimension of the caches must be 16, got {chunk}")
+    _check(chunk == 16, lambda: f"paged_attention: last dimension of the caches must be 16, got {chunk}")
     _check(value_cache.shape == key_cache.shape, "paged_attention: key_cache and value_cache must have the same shape")
     _check(
         head_dim > 0 and (nh16 * 16) % head_dim == 0 and nh16 * 16 >= head_dim,
-        f"paged_attention: cache rows ({nh16 * 16} halfs) must hold whole heads of {head_dim}",
+        lambda: f"paged_attention: cache rows ({nh16 * 16} halfs) must hold whole heads of {head_dim}",
     )
     num_kv_heads = nh16 * 16 // head_dim
     _check(
         num_heads % num_kv_heads == 0,
-        f"paged_attention: num_heads ({num_heads}) must be a multiple of num_kv_heads ({num_kv_heads})",
+        lambda: f"paged_attention: num_heads ({num_heads}) must be a multiple of num_kv_heads ({num_kv_heads})",
     )
     _check(
         block_tables.size(0) == bs and context_lens.size(0) == bs,
@@ -384,7 +394,7 @@ def paged_attention(q, key_cache, value_cache, block_tables, context_lens):
     ws_bytes = _lib.aops_paged_attention_workspace(bs, num_heads, num_kv_heads, head_dim, block_size, max_blocks)
     _check(
         ws_bytes > 0,
-        f"paged_attention: unsupported shape (head_dim={head_dim}, block_size={block_size}); "
+        lambda: f"paged_attention: unsupported shape (head_dim={head_dim}, block_size={block_size}); "
         "head_dim must be a multiple of 16 up to 256",
     )
     workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
@@ -408,25 +418,25 @@ def rope_reshape_and_cache(q, k, v, position_ids, cos_cache, sin_cache, key_cach
     _check(
         q.dim() == 3 and k.dim() == 3 and v.dim() == 3 and position_ids.dim() == 1 and cos_cache.dim() == 2
         and sin_cache.dim() == 2 and key_cache.dim() == 4 and value_cache.dim() == 4 and slot_indices.dim() == 1,
-        f"{name}: q, k, v must be 3D, position_ids and slot_indices 1D, cos_cache and sin_cache 2D, caches 4D",
+        lambda: f"{name}: q, k, v must be 3D, position_ids and slot_indices 1D, cos_cache and sin_cache 2D, caches 4D",
     )
     _check(
         all(t.is_contiguous() for t in (q, k, v, position_ids, cos_cache, sin_cache, key_cache, value_cache, slot_indices)),
-        f"{name}: all input tensors must be contiguous",
+        lambda: f"{name}: all input tensors must be contiguous",
     )
     bs, num_heads, head_dim = q.shape
     num_kv_heads = k.size(1)
     _check(k.size(0) == bs and k.size(2) == head_dim and v.shape == k.shape,
-           f"{name}: k and v must be [bs, num_kv_heads, head_dim] matching q")
+           lambda: f"{name}: k and v must be [bs, num_kv_heads, head_dim] matching q")
     _check(position_ids.size(0) == bs and slot_indices.size(0) == bs,
-           f"{name}: position_ids and slot_indices must have one entry per token")
-    _check(head_dim % 16 == 0, f"{name}: head_dim must be a multiple of 16, got {head_dim}")
+           lambda: f"{name}: position_ids and slot_indices must have one entry per token")
+    _check(head_dim % 16 == 0, lambda: f"{name}: head_dim must be a multiple of 16, got {head_dim}")
     _check(cos_cache.size(1) == head_dim // 2 and sin_cache.shape == cos_cache.shape,
-           f"{name}: cos_cache and sin_cache must be [max_position, head_dim/2]")
+           lambda: f"{name}: cos_cache and sin_cache must be [max_position, head_dim/2]")
     num_blocks, nh16, block_size, chunk = key_cache.shape
     _check(
         chunk == 16 and nh16 * 16 == num_kv_heads * head_dim and value_cache.shape == key_cache.shape,
-        f"{name}: caches must be [num_blocks, num_kv_heads*head_dim/16, block_size, 16], got "
+        lambda: f"{name}: caches must be [num_blocks, num_kv_heads*head_dim/16, block_size, 16], got "
         f"{tuple(key_cache.shape)} and {tuple(value_cache.shape)}",
     )
     _require_device(
@@ -441,11 +451,11 @@ def rope_reshape_and_cache(q, k, v, position_ids, cos_cache, sin_cache, key_cach
     out_q = torch.empty_like(q)
     out_k = torch.empty_like(k) if return_k else None
     if norm:
-        _check(q_norm_weight is not None and k_norm_weight is not None, f"{name}: give both norm weights or none")
+        _check(q_norm_weight is not None and k_norm_weight is not None, lambda: f"{name}: give both norm weights or none")
         _check(q_norm_weight.shape == (head_dim,) and k_norm_weight.shape == (head_dim,)
                and q_norm_weight.is_contiguous() and k_norm_weight.is_contiguous(),
-               f"{name}: norm weights must be contiguous [head_dim] tensors")
-        _check(head_dim in (16, 32, 64, 128, 256), f"{name}: the fused norm needs head_dim 16, 32, 64, 128 or 256, got {head_dim}")
+               lambda: f"{name}: norm weights must be contiguous [head_dim] tensors")
+        _check(head_dim in (16, 32, 64, 128, 256), lambda: f"{name}: the fused norm needs head_dim 16, 32, 64, 128 or 256, got {head_dim}")
         _require_device(name, {"q_norm_weight": (q_norm_weight, torch.float16), "k_norm_weight": (k_norm_weight, torch.float16)})
         code = _lib.aops_qknorm_rope_reshape_and_cache_f16(
             _ptr(q), _ptr(k), _ptr(v), _ptr(q_norm_weight), _ptr(k_norm_weight), float(epsilon), _ptr(position_ids),
@@ -469,21 +479,21 @@ def grouped_matmul_swiglu_gather(x, sorted_idx, topk, w, group_list):
     copy: the kernel reads row ``sorted_idx[j] // topk`` of ``x`` for sorted row ``j``."""
     name = "grouped_matmul_swiglu_gather"
     _check(x.dim() == 2 and x.is_contiguous() and sorted_idx.dim() == 1 and sorted_idx.is_contiguous(),
-           f"{name}: x must be 2D, sorted_idx 1D, both contiguous")
+           lambda: f"{name}: x must be 2D, sorted_idx 1D, both contiguous")
     _check(topk > 0 and sorted_idx.numel() == x.size(0) * topk,
-           f"{name}: sorted_idx must have tokens*topk entries, got {sorted_idx.numel()} for {x.size(0)} tokens, topk {topk}")
+           lambda: f"{name}: sorted_idx must have tokens*topk entries, got {sorted_idx.numel()} for {x.size(0)} tokens, topk {topk}")
     rows = sorted_idx.numel()
     dim = x.size(1)
     if dim % 128 != 0 or dim < 256 or x.size(0) * dim >= 2 ** 32:
         return grouped_matmul_swiglu(moe_gather(x, sorted_idx, group_list, topk), w, group_list)
     # the remaining checks are those of grouped_matmul on the (virtual) gathered matrix
-    _check(w.dim() == 3 and group_list.dim() == 1 and group_list.is_contiguous(), f"{name}: w must be 3D, group_list 1D")
-    _check(dim == w.size(1), f"{name}: last dimension of x must match second dimension of w, got {dim} and {w.size(1)}")
-    _check(w.stride(1) == 1 and w.stride(2) == dim, f"{name}: w must be K-major order, got strides {tuple(w.stride())}")
-    _check(w.size(2) % 64 == 0, f"{name}: third dimension of w must be a multiple of 64, got {w.size(2)}")
+    _check(w.dim() == 3 and group_list.dim() == 1 and group_list.is_contiguous(), lambda: f"{name}: w must be 3D, group_list 1D")
+    _check(dim == w.size(1), lambda: f"{name}: last dimension of x must match second dimension of w, got {dim} and {w.size(1)}")
+    _check(w.stride(1) == 1 and w.stride(2) == dim, lambda: f"{name}: w must be K-major order, got strides {tuple(w.stride())}")
+    _check(w.size(2) % 64 == 0, lambda: f"{name}: third dimension of w must be a multiple of 64, got {w.size(2)}")
     num_experts, inner_dim = w.size(0), w.size(2)
-    _check(num_experts <= 1 or w.stride(0) == dim * inner_dim, f"{name}: experts of w must be densely packed")
-    _check(group_list.size(0) == num_experts, f"{name}: group_list must have one entry per expert")
+    _check(num_experts <= 1 or w.stride(0) == dim * inner_dim, lambda: f"{name}: experts of w must be densely packed")
+    _check(group_list.size(0) == num_experts, lambda: f"{name}: group_list must have one entry per expert")
     _require_device(name, {"x": (x, torch.float16), "w": (w, torch.float16), "group_list": (group_list, torch.int64),
                            "sorted_idx": (sorted_idx, torch.int32)})
     y = torch.empty((rows, inner_dim // 2), dtype=x.dtype, device=x.device)
@@ -496,7 +506,7 @@ def grouped_matmul_swiglu_gather(x, sorted_idx, topk, w, group_list):
 def moe_sort(topk_ids, num_experts):
     """Stable sort of the flattened routing by expert: (sorted_idx, inverse_idx, group_list)."""
     _check(topk_ids.dim() in (1, 2) and topk_ids.is_contiguous(), "moe_sort: topk_ids must be a contiguous 1D or 2D tensor")
-    _check(0 < num_experts <= 4095, f"moe_sort: num_experts must be in 1..4095, got {num_experts}")
+    _check(0 < num_experts <= 4095, lambda: f"moe_sort: num_experts must be in 1..4095, got {num_experts}")
     _require_device("moe_sort", {"topk_ids": (topk_ids, torch.int32)})
     n = topk_ids.numel()
     dev = topk_ids.device
@@ -504,7 +514,7 @@ def moe_sort(topk_ids, num_experts):
     inverse_idx = torch.empty(n, dtype=torch.int32, device=dev)
     group_list = torch.empty(num_experts, dtype=torch.int64, device=dev)
     ws_bytes = _lib.aops_moe_sort_workspace(n, num_experts)
-    _check(ws_bytes > 0, f"moe_sort: unsupported size n={n}, num_experts={num_experts}")
+    _check(ws_bytes > 0, lambda: f"moe_sort: unsupported size n={n}, num_experts={num_experts}")
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     code = _lib.aops_moe_sort_i32(_ptr(topk_ids), n, num_experts, _ptr(sorted_idx), _ptr(inverse_idx), _ptr(group_list),
                                   _ptr(ws), ws_bytes, _stream(dev))
@@ -517,8 +527,8 @@ def moe_gather(x, sorted_idx, group_list, topk):
     _check(x.dim() == 2 and x.is_contiguous() and sorted_idx.dim() == 1 and sorted_idx.is_contiguous()
            and group_list.dim() == 1 and group_list.is_contiguous(), "moe_gather: x must be 2D, sorted_idx and group_list 1D, all contiguous")
     _check(topk > 0 and sorted_idx.numel() == x.size(0) * topk,
-           f"moe_gather: sorted_idx must have tokens*topk entries, got {sorted_idx.numel()} for {x.size(0)} tokens, topk {topk}")
-    _check(x.size(1) % 8 == 0, f"moe_gather: hidden must be a multiple of 8, got {x.size(1)}")
+           lambda: f"moe_gather: sorted_idx must have tokens*topk entries, got {sorted_idx.numel()} for {x.size(0)} tokens, topk {topk}")
+    _check(x.size(1) % 8 == 0, lambda: f"moe_gather: hidden must be a multiple of 8, got {x.size(1)}")
     _require_device("moe_gather", {"x": (x, torch.float16), "sorted_idx": (sorted_idx, torch.int32),
                                    "group_list": (group_list, torch.int64)})
     n = sorted_idx.numel()
@@ -536,8 +546,8 @@ def moe_combine(y, inverse_idx, topk_weights, topk_ids, num_experts):
            "moe_combine: y must be 2D, topk_weights and topk_ids [tokens, topk], all contiguous")
     tokens, topk = topk_weights.shape
     _check(y.size(0) == tokens * topk and inverse_idx.numel() == tokens * topk,
-           f"moe_combine: y and inverse_idx must have tokens*topk rows, got {y.size(0)} and {inverse_idx.numel()}")
-    _check(y.size(1) % 8 == 0, f"moe_combine: hidden must be a multiple of 8, got {y.size(1)}")
+           lambda: f"moe_combine: y and inverse_idx must have tokens*topk rows, got {y.size(0)} and {inverse_idx.numel()}")
+    _check(y.size(1) % 8 == 0, lambda: f"moe_combine: hidden must be a multiple of 8, got {y.size(1)}")
     _require_device("moe_combine", {"y": (y, torch.float16), "inverse_idx": (inverse_idx, torch.int32),
                                     "topk_weights": (topk_weights, torch.float32), "topk_ids": (topk_ids, torch.int32)})
     out = torch.empty((tokens, y.size(1)), dtype=y.dtype, device=y.device)
