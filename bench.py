@@ -630,7 +630,12 @@ def main():
     def run(tag, fn):
         if allops or tag in want:
             t0 = time.perf_counter()
-            res = fn()
+            try:
+                res = fn()
+            except Exception as exc:  # the headline line must still be printed; the failure goes into it
+                log(f"[bench] {tag} FAILED: {exc!r}")
+                res = {"op_group": tag, "error": repr(exc)[:400]}
+                torch.cuda.synchronize()
             res = res if isinstance(res, list) else [res]
             per_op.extend(res)
             for r in res:
