@@ -96,3 +96,36 @@ def test_decode_step_and_expert_mlp_in_one_graph(ops, dev):
     # and the eager results themselves are right (attention of the last seed against the oracle)
     ref = R.paged_attention_ref(want[2].cpu(), kc.cpu(), vc.cpu(), fresh["bt"], fresh["ctx"])
     torch.testing.assert_close(want[4].cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+
+
+def test_two_streams_concurrently(ops, dev):
+    """Entry points keep no device-side state between calls, so independent work on two streams may overlap:
+    a grouped matmul chain on one stream and decode attention on the other, several rounds, against the same
+    work done alone."""
+    import ascend910a_extras.fused as fused
+
+    g = torch.Generator().manual_seed(21)
+    E, K, I, rows = 32, 512, 256, 8192
+    xs = torch.randn(rows, K, generator=g).half().to(dev)
+    w1 = (0.05 * torch.randn(E, 2 * I, K, generator=g)).half().to(dev).transpose(1, 2)
+    gl = R.make_group_list(torch.randint(0, E, (rows,), generator=g), E).to(dev)
+    B, Hq, Hkv, D, P, NB = 16, 32, 8, 128, 128, 160
+    kc = torch.randn(NB, Hkv * D // 16, P, 16, generator=g).half().to(dev)
+    vc = torch.randn(NB, Hkv * D // 16, P, 16, generator=g).half().to(dev)
+    bt = torch.randperm(NB, generator=g).int().reshape(B, NB // B).to(dev)
+    cl = torch.randint(1, P * (NB // B) + 1, (B,), generator=g, dtype=torch.int32).to(dev)
+    q = torch.randn(B, Hq, D, generator=g).half().to(dev)
+    want_h = fused.grouped_matmul_swiglu(xs, w1, gl)
+    want_o = ops.paged_attention(q, kc, vc, bt, cl)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    for _ in range(5):
+        with torch.cuda.stream(s1):
+            h = fused.grouped_matmul_swiglu(xs, w1, gl)
+            h2 = ops.swiglu(ops.grouped_matmul(xs, w1, gl))
+        with torch.cuda.stream(s2):
+            o = ops.paged_attention(q, kc, vc, bt, cl)
+            o2 = ops.paged_attention(q, kc, vc, bt, cl)
+        torch.cuda.synchronize()
+        assert torch.equal(h, want_h) and torch.equal(o, want_o) and torch.equal(o2, want_o)
+        torch.testing.assert_close(h2.float(), want_h.float(), rtol=2e-2, atol=2e-2)
