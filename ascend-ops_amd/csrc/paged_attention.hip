@@ -161,7 +161,7 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ context_lens, float* __restrict__ part_o,
     float* __restrict__ part_ml, f16* __restrict__ out, int num_kv_heads, int block_size, int max_blocks_per_seq,
-    int chunk_tokens, int max_splits, float scale_log2) {
+    int chunk_tokens, int max_splits, float scale_log2, int num_blocks) {
   const int split = blockIdx.x;
   const int g = blockIdx.y;
   // Workgroups are handed out in index order, so they take the sequences longest first: with
@@ -232,7 +232,8 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
   auto page_offset = [&](int step) -> int64_t {
     const int tok = chunk_start + step * kPaStep;  // first token of the step (wave uniform)
     const int blk = tok / block_size;
-    const int64_t page = table[blk];
+    // a table entry outside the cache reads the nearest page instead of faulting
+    const int64_t page = min(max(table[blk], 0), num_blocks - 1);
     return page * page_elems + head_off + (int64_t)(tok - blk * block_size) * 16;
   };
 
@@ -351,18 +352,18 @@ template <int G>
 static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t* bt,
                       const int32_t* cl, f16* o, float* part_o, float* part_ml, int bs,
                       int num_heads, int num_kv_heads, int block_size, int max_blocks_per_seq,
-                      PaChunking ch, hipStream_t s) {
+                      PaChunking ch, hipStream_t s, int num_blocks) {
   const float scale_log2 = kLog2e / __builtin_sqrtf((float)kPaD);
   dim3 grid((unsigned)ch.max_splits, (unsigned)num_kv_heads, (unsigned)bs);
   if (ch.max_splits == 1) {
     pa_decode_partial<G, true><<<grid, kPaWaves * kWave, 0, s>>>(
         q, kc, vc, bt, cl, part_o, part_ml, o, num_kv_heads, block_size, max_blocks_per_seq,
-        ch.chunk_tokens, ch.max_splits, scale_log2);
+        ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks);
     return;
   }
   pa_decode_partial<G, false><<<grid, kPaWaves * kWave, 0, s>>>(
       q, kc, vc, bt, cl, part_o, part_ml, o, num_kv_heads, block_size, max_blocks_per_seq,
-      ch.chunk_tokens, ch.max_splits, scale_log2);
+      ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks);
   dim3 mgrid((unsigned)num_heads, (unsigned)bs);
   pa_decode_merge<<<mgrid, kPaD, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
                                          ch.max_splits);
@@ -379,7 +380,8 @@ __global__ __launch_bounds__(4 * kWave) void pa_decode_generic(
     const f16* __restrict__ q, const f16* __restrict__ key_cache,
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ context_lens, f16* __restrict__ out, int num_heads,
-    int num_kv_heads, int head_dim, int block_size, int max_blocks_per_seq, float scale_log2) {
+    int num_kv_heads, int head_dim, int block_size, int max_blocks_per_seq, float scale_log2,
+    int num_blocks) {
   constexpr int kPerLane = kPaGenericMaxD / kWave;
   const int h = blockIdx.x;
   const int b = blockIdx.y;
@@ -404,7 +406,7 @@ __global__ __launch_bounds__(4 * kWave) void pa_decode_generic(
   float m = kNegBig, l = 0.f;
   for (int j = wave; j < context_len; j += 4) {
     const int blk = j / block_size;
-    const int64_t base = (int64_t)table[blk] * row_chunks * block_size * 16 +
+    const int64_t base = (int64_t)min(max(table[blk], 0), num_blocks - 1) * row_chunks * block_size * 16 +
                          (int64_t)(j - blk * block_size) * 16;
     float part = 0.f, vf[kPerLane];
 #pragma unroll
@@ -483,10 +485,11 @@ extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
                                         int64_t block_size, int64_t max_blocks_per_seq,
                                         int64_t num_blocks, void* stream) {
   using namespace aops;
-  (void)num_blocks;
-  if (!pa_args_valid(bs, num_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq))
+  if (!pa_args_valid(bs, num_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq) ||
+      num_blocks < 0 || num_blocks > 0x7fffffff)
     return AOPS_ERR_INVALID_ARGUMENT;
   if (bs == 0) return AOPS_OK;
+  if (num_blocks == 0) return AOPS_ERR_INVALID_ARGUMENT;  // sequences but no cache to read
   if (!q || !key_cache || !value_cache || !block_tables || !context_lens || !o)
     return AOPS_ERR_INVALID_ARGUMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -500,7 +503,7 @@ extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
     pa_decode_generic<<<grid, 4 * kWave, 0, s>>>(qp, kc, vc, block_tables, context_lens, op,
                                                  (int)num_heads, (int)num_kv_heads, (int)head_dim,
                                                  (int)block_size, (int)max_blocks_per_seq,
-                                                 scale_log2);
+                                                 scale_log2, (int)num_blocks);
     return record_launch_status(hipGetLastError());
   }
   const size_t need = aops_paged_attention_workspace(bs, num_heads, num_kv_heads, head_dim,
@@ -513,7 +516,7 @@ extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
   case G:                                                                                      \
     pa_launch<G>(qp, kc, vc, block_tables, context_lens, op, part_o, part_ml, (int)bs,         \
                  (int)num_heads, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq,  \
-                 ch, s);                                                                       \
+                 ch, s, (int)num_blocks);                                                      \
     break;
   switch (num_heads / num_kv_heads) {
     AOPS_PA_CASE(1)

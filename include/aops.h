@@ -218,7 +218,8 @@ int aops_moe_combine_f16(const void* y, const int32_t* inverse_idx, const float*
  * be a multiple of 16 up to 256.  head_dim 128 with block_size a multiple of 32 and
  * num_heads/num_kv_heads in {1, 2, 4, 8, 16} runs on the matrix cores; every other shape takes a
  * generic, untuned kernel.  A sequence with context_len <= 0 gets zeros; a context_len beyond
- * max_blocks_per_seq*block_size is cut there.  Block-table entries are not range-checked.
+ * max_blocks_per_seq*block_size is cut there.  Block-table entries outside [0, num_blocks) are
+ * clamped into it (garbage in, garbage out, no fault).
  * Replaces aclnnPagedAttentionExGetWorkspaceSize + aclnnPagedAttentionEx
  * (reference csrc/ffi/ops.cpp:454-461).
  */

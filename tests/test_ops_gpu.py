@@ -438,6 +438,24 @@ def test_paged_attention(ops, dev, B, Hq, Hkv, P, lens):
     assert (o.float() - ref.float()).abs().max() < 2e-3
 
 
+@pytest.mark.parametrize("D,P,Hq,Hkv", [(128, 128, 32, 8), (64, 16, 6, 2)])
+def test_paged_attention_clamps_block_table_entries(ops, dev, D, P, Hq, Hkv):
+    """Block-table entries outside the cache are clamped into it (both kernels): the sequences with valid tables are
+    unaffected, the sequence with bad entries equals the result for the clamped table."""
+    lens = [3 * P + 5, 2 * P, P + 1]
+    q, kc, vc, bt, cl = _paged_case(3, Hq, Hkv, D, P, lens, seed=4)
+    NB = kc.size(0)
+    bad = bt.clone()
+    bad[1, 0] = NB + 1000
+    bad[1, 1] = -7
+    o = ops.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), bad.to(dev), cl.to(dev)).cpu()
+    clamped = bad.clone().clamp_(0, NB - 1)
+    ref = R.paged_attention_ref(q, kc, vc, clamped, cl)
+    torch.testing.assert_close(o.float(), ref.float(), **TOL)
+    good = R.paged_attention_ref(q, kc, vc, bt, cl)
+    torch.testing.assert_close(o[[0, 2]].float(), good[[0, 2]].float(), **TOL)
+
+
 def test_paged_attention_batch_larger_than_a_wave(ops, dev):
     """More than 64 sequences: the longest-first ordering of the workgroups (one length per lane) is off and the
     sequences are taken in index order; several chunks per sequence when the batch alone fills the chip."""
