@@ -230,7 +230,8 @@ __global__ __launch_bounds__(256) void moe_gather_kernel(const f16* __restrict__
   const int64_t j = i / vec_per_row;
   if (j >= rows) return;
   const uint32_t c = (uint32_t)(i - j * vec_per_row);
-  const int64_t src = sorted_idx[j] / topk;
+  // an index outside the routing table reads the last token instead of faulting
+  const int64_t src = min(max((int64_t)sorted_idx[j], (int64_t)0), n - 1) / topk;
   st128_stream(out + (j * vec_per_row + c) * 8, ld128(x + (src * vec_per_row + c) * 8));
 }
 
@@ -259,7 +260,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
       const bool ok = k < topk && id >= 0 && id < num_experts;
       wgt[j] = ok ? weights[f] : 0.f;
       // rows of ids that are not routed are never written: read row 0 instead and drop the value
-      const int64_t row = ok ? inverse_idx[f] : 0;
+      const int64_t row = ok ? min(max((int64_t)inverse_idx[f], (int64_t)0), tokens * topk - 1) : 0;
       v[j] = ld128_stream(y + (row * vec_per_row + c) * 8);
       if (!ok) v[j] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     }
