@@ -376,6 +376,42 @@ def _gmm_swiglu_gather_entry(L, dev, w_storage, tokens, topk):
                  "extension: replaces moe_gather + gate_up + swiglu; one weight set, so the weights are re-read from HBM every launch but x (17 MB) stays cached")
 
 
+def _moe_mlp_entry(dev, w1_storage, w2_storage, tokens, topk):
+    """The whole routed expert MLP of configs[3] through the extension API (sort -> gate_up with gather and SwiGLU
+    -> down -> combine), captured in one HIP graph: what the operators add up to for a caller."""
+    import torch
+    import ascend910a_extras.moe as moe
+
+    E, N1, K = w1_storage.shape
+    torch.manual_seed(3)
+    x = torch.randn(tokens, K).half().to(dev)
+    logits = torch.randn(tokens, E)
+    wts, ids = torch.topk(torch.softmax(logits, -1), topk, dim=-1)
+    wts = (wts / wts.sum(-1, keepdim=True)).float().to(dev)
+    ids = ids.int().to(dev)
+    w1 = w1_storage.to(dev).transpose(1, 2)
+    w2 = w2_storage.to(dev).transpose(1, 2)
+    for _ in range(2):
+        out = moe.moe_mlp(x, ids, wts, w1, w2)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = moe.moe_mlp(x, ids, wts, w1, w2)
+    graph.replay()
+    torch.cuda.synchronize()
+    trials = []
+    for _ in range(5):
+        trials.append(_events_ms(graph.replay, 10) * 1e3 / 10)
+    trials.sort()
+    flops = 2 * tokens * topk * K * N1 + 2 * tokens * topk * (N1 // 2) * K
+    e = {"op": "moe_mlp", "config": "4: routed expert MLP end to end (extension, five launches in one graph)",
+         "shape": f"x [{tokens},{K}], top-{topk} of {E} experts, inter {N1 // 2}", "bound": "mfma",
+         "algorithmic_flops": flops, "gpu_us": round(trials[len(trials) // 2], 3), "gpu_us_min": round(trials[0], 3)}
+    e["TFLOPs"] = round(flops / e["gpu_us"] / 1e6, 1)
+    e["mfma_frac"] = round(e["TFLOPs"] / MFMA_F16_PEAK_TFLOPS, 4)
+    return e
+
+
 def _moe_glue_entries(L, dev, E, hidden, tokens, topk):
     """Routing glue of the expert MLP at the configs[3] shape (extension, no reference operator): device-side
     stable sort -> group_list, row gather, weighted combine.  Checked against the oracle in tests/test_moe_gpu.py."""
@@ -435,6 +471,7 @@ def bench_moe(L, ops, R, dev, cpu):
     out.append(e1)
     e_fused = _gmm_swiglu_entry(L, ops, dev, "4: MoE gate_up + activation, fused", x, w1, gl, h_dev)
     e_gather = _gmm_swiglu_gather_entry(L, dev, w1, tokens, topk)
+    e_layer = _moe_mlp_entry(dev, w1, w2, tokens, topk)
     del w1
     h = ops.swiglu(h_dev)
     # swiglu at the MoE shape
@@ -455,6 +492,7 @@ def bench_moe(L, ops, R, dev, cpu):
     out.append(e2)
     out.append(e_fused)
     out.append(e_gather)
+    out.append(e_layer)
     out.extend(_moe_glue_entries(L, dev, E, hidden, tokens, topk))
     tot_flops = e1["algorithmic_flops"] + e2["algorithmic_flops"]
     tot_us = e1["gpu_us"] + e2["gpu_us"]
