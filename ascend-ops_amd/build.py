@@ -100,6 +100,25 @@ def build_library(force: bool = True, verbose: bool = False) -> Path:
     return lib
 
 
+def emit_assembly(out_dir: Path, sources=None) -> list:
+    """Writes the compiler's gfx950 assembly of the given sources (default: all) into ``out_dir``, built
+    with the flags of the library, and returns the paths.  Used to inspect what the compiler made of the
+    kernels (register counts, scheduling, the distance between matrix-core results and their readers)."""
+    hipcc = _hipcc()
+    out_dir = Path(out_dir)
+    out_dir.mkdir(parents=True, exist_ok=True)
+    flags = [f for f in HIPCC_FLAGS if f != "-fPIC"]
+
+    def one(name: str) -> Path:
+        out = out_dir / (name + ".s")
+        _run([hipcc, *flags, "--cuda-device-only", "-S", str(CSRC / name), "-o", str(out)])
+        return out
+
+    names = list(sources or SOURCES)
+    with ThreadPoolExecutor(max_workers=min(8, len(names))) as pool:
+        return list(pool.map(one, names))
+
+
 if __name__ == "__main__":
     path = build_library(force="--force" in sys.argv, verbose=True)
     print(path)

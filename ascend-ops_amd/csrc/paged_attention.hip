@@ -99,6 +99,13 @@ __device__ __forceinline__ void pa_scores(const PaRegs& k, const f16x8 (&qreg)[4
 #pragma unroll
     for (int s = 0; s < 4; ++s)
       sacc[g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(k[g][s], qreg[s], sacc[g], 0, 0, 0);
+  // A matrix-core result may only be read six wait states after its instruction (four passes plus
+  // two).  The compiler keeps that distance inside a basic block, but when it places the
+  // accumulators in AGPRs and a taken branch (the "no further step" case of the caller) lies between
+  // the last product and the first v_accvgpr_read, it emits the read two wait states after the
+  // product and the last score of every step comes back stale.  Pinning the accumulators to VGPRs
+  // here and spending eight idle cycles keeps the distance whatever the block layout.
+  asm volatile("s_nop 7" : "+v"(sacc[0]), "+v"(sacc[1]));
 #pragma unroll
   for (int g = 0; g < 2; ++g)
 #pragma unroll
