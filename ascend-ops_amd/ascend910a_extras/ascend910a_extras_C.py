@@ -51,6 +51,8 @@ _SIGNATURES = {
     "aops_moe_gather_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_moe_combine_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "aops_paged_attention_workspace": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64]),
+    "aops_matmul_nt_workspace": (_sz, [_i64, _i64, _i64]),
+    "aops_matmul_nt_ws_f16": (ctypes.c_int, [_vp, _vp, _vp, _vp, _sz, _i64, _i64, _i64, _vp]),
     "aops_paged_attention_f16": (
         ctypes.c_int,
         [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _vp],
@@ -225,11 +227,25 @@ def grouped_matmul(x, w, group_list):
     num_tokens, dim = x.shape
     num_experts, inner_dim = w.size(0), w.size(2)
     y = torch.empty((num_tokens, inner_dim), dtype=x.dtype, device=x.device)
+    if num_experts == 1 and _dense_split_k(x, w, y, num_tokens, dim, inner_dim, "grouped_matmul"):
+        return y  # one expert, few rows, long k: the dense kernel with a split k range (all rows computed)
     code = _lib.aops_grouped_matmul_f16(
         _ptr(x), _ptr(w), _ptr(group_list), _ptr(y), num_tokens, dim, num_experts, inner_dim, _stream(x.device)
     )
     _status("grouped_matmul", code)
     return y
+
+
+def _dense_split_k(x, w, y, m, k, n, name) -> bool:
+    """Runs y = x @ w^T through the split-k entry point if the library wants a workspace for the shape
+    (few rows, long k); returns False, having done nothing, otherwise."""
+    ws_bytes = _lib.aops_matmul_nt_workspace(m, k, n)
+    if ws_bytes == 0:
+        return False
+    workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+    code = _lib.aops_matmul_nt_ws_f16(_ptr(x), _ptr(w), _ptr(y), _ptr(workspace), ws_bytes, m, k, n, _stream(x.device))
+    _status(name, code)
+    return True
 
 
 def matmul(x, w):
@@ -245,6 +261,8 @@ def matmul(x, w):
     _check(k % 64 == 0 and n % 64 == 0, lambda: f"matmul: k and n must be multiples of 64, got k={k} and n={n}")
     _require_device("matmul", {"x": (x, torch.float16), "w": (w, torch.float16)})
     y = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    if m > 0 and _dense_split_k(x, w, y, m, k, n, "matmul"):
+        return y
     code = _lib.aops_matmul_nt_f16(_ptr(x), _ptr(w), _ptr(y), m, k, n, _stream(x.device))
     _status("matmul", code)
     return y

@@ -283,4 +283,12 @@ int gmm_launch_persistent(bool swiglu, const f16* x, const f16* w, const int64_t
                           int64_t rows, int k, int num_experts, int n, hipStream_t stream,
                           const int32_t* row_idx, int idx_div, int64_t x_rows);
 
+// Dense [m, k] x [n, k]^T with the k range split over several workgroups per output tile and a
+// second kernel adding the partial results: for few rows and a long k, where whole-k tiles would
+// leave most CUs without work.  gmm_splitk_workspace returns the bytes of fp32 scratch the call
+// needs on the current device, 0 when splitting does not pay for the shape.
+size_t gmm_splitk_workspace(int64_t m, int64_t k, int64_t n);
+int gmm_launch_splitk(const f16* x, const f16* w, f16* y, float* workspace, size_t workspace_bytes,
+                      int64_t m, int k, int n, hipStream_t stream);
+
 }  // namespace aops

@@ -88,6 +88,30 @@ extern "C" int aops_matmul_nt_f16(const void* x, const void* w, void* y, int64_t
   return aops_grouped_matmul_impl(x, w, nullptr, y, m, k, 1, n, stream);
 }
 
+static bool matmul_nt_args_valid(int64_t m, int64_t k, int64_t n) {
+  return m >= 0 && k > 0 && n > 0 && k % 64 == 0 && n % 64 == 0 && m <= 0x7fffffff - 4096 &&
+         k <= (1 << 22) && n <= 0x7fffffff;
+}
+
+extern "C" size_t aops_matmul_nt_workspace(int64_t m, int64_t k, int64_t n) {
+  if (!matmul_nt_args_valid(m, k, n) || m == 0) return 0;
+  if (getenv("AOPS_GMM_VARIANT")) return 0;  // a forced kernel choice also switches the k split off
+  return aops::gmm_splitk_workspace(m, k, n);
+}
+
+extern "C" int aops_matmul_nt_ws_f16(const void* x, const void* w, void* y, void* workspace,
+                                     size_t workspace_bytes, int64_t m, int64_t k, int64_t n,
+                                     void* stream) {
+  if (!matmul_nt_args_valid(m, k, n)) return AOPS_ERR_INVALID_ARGUMENT;
+  if (m == 0) return AOPS_OK;
+  if (!x || !w || !y) return AOPS_ERR_INVALID_ARGUMENT;
+  if (aops_matmul_nt_workspace(m, k, n) == 0)
+    return aops_grouped_matmul_impl(x, w, nullptr, y, m, k, 1, n, stream);
+  return aops::gmm_launch_splitk(static_cast<const aops::f16*>(x), static_cast<const aops::f16*>(w),
+                                 static_cast<aops::f16*>(y), static_cast<float*>(workspace),
+                                 workspace_bytes, m, (int)k, (int)n, static_cast<hipStream_t>(stream));
+}
+
 extern "C" int aops_grouped_matmul_swiglu_gather_f16(const void* x, const int32_t* row_idx,
                                                      int64_t idx_div, int64_t x_rows, const void* w,
                                                      const int64_t* group_list, void* y, int64_t rows,

@@ -247,6 +247,61 @@ __global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
   }
 }
 
+// Writes a workgroup's accumulators (acc[i][j][4g+e] of wave (wm, wn): row 32*(wm+2i) + lane%32,
+// column wn*32*NB + 32j + 8g + 4*(lane/32) + e of the tile) as fp16 through LDS, one pass per pair
+// of wave columns, so that y is written in 16-byte pieces along its rows.  All waves of the
+// workgroup call it after a barrier; `smem` must hold BM x 64*NB halfs.
+template <int MB, int NB, int WN>
+__device__ __forceinline__ void gmm_store_tile(const f32x16 (&acc)[MB][NB], f16* smem, f16* __restrict__ y,
+                                               int row_begin, int tile_rows, int n_tile, int n) {
+  constexpr int kWaves = 2 * WN;
+  constexpr int BN = 32 * NB * WN;
+  constexpr int kThreads = kWaves * kWave;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave / WN;
+  const int wn = wave % WN;
+  const int fm = lane & 31;
+  const int fq = lane >> 5;
+  f16* sc = smem;
+  constexpr int kPassCols = 64 * NB;  // columns of two wave columns
+  constexpr int kSwz = (kPassCols / 8 < 16 ? kPassCols / 8 : 16) - 1;
+  constexpr int kChunksPerRow = kPassCols / 8;
+  constexpr int kRowsPerStorePass = kThreads / kChunksPerRow;
+#pragma unroll
+  for (int pass = 0; pass < WN / 2; ++pass) {
+    if (wn / 2 == pass) {
+#pragma unroll
+      for (int i = 0; i < MB; ++i) {
+        const int m = 32 * (wm + 2 * i) + fm;
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            f16x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = (f16)acc[i][j][4 * g + e];
+            const int piece = ((wn & 1) * 32 * NB + 32 * j + 8 * g + 4 * fq) >> 2;
+            *reinterpret_cast<f16x4*>(&sc[m * kPassCols + ((piece ^ ((m & kSwz) << 1)) << 2)]) = v;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    const int c16 = tid % kChunksPerRow;
+    const int col = n_tile * BN + pass * kPassCols + c16 * 8;
+    if (col < n) {
+      for (int m = tid / kChunksPerRow; m < tile_rows; m += kRowsPerStorePass) {
+        const f16x8 v =
+            *reinterpret_cast<const f16x8*>(&sc[m * kPassCols + ((c16 ^ (m & kSwz)) << 3)]);
+        st128(y + (int64_t)(row_begin + m) * n + col, v);
+      }
+    }
+    if (pass + 1 < WN / 2) __syncthreads();
+  }
+}
+
 // Same tiling and MFMA work as grouped_matmul_kernel, but both operand tiles travel HBM -> LDS
 // directly (global_load_lds_dwordx4: 64 lanes deposit 64 consecutive 16-byte chunks), so the k
 // loop holds no staging registers and issues no LDS writes.  Because a lane cannot choose where
@@ -257,10 +312,21 @@ __global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
 //   then      : wait for this wave's copies of tile kt+1, barrier (tile kt+1 complete for
 //               everyone, nobody reads stage kt&1 any more)
 //   step 3    : MFMAs | fragment reads of step 0 of tile kt+1 | copies of tile kt+2 into stage kt&1
-template <int MB, int NB, int WN>
+//
+// SPLITK = true is the dense form for few rows and a long k (one group, group_list unused): workgroup
+// blockIdx.x computes output tile blockIdx.x / splits over the k tiles of split blockIdx.x % splits
+// (workgroup i runs on XCD i % 8, so with 8 splits every XCD reads one k range of x and keeps it in
+// its L2) and leaves its fp32 accumulators in `partial` in register order: for (split, tile, wave)
+// a block of MB*NB*4 rows of 64 float4, row (i*NB + j)*4 + g holding acc[i][j][4g..4g+3] of every
+// lane, so that each store instruction writes 1 KiB of consecutive bytes.  matmul_splitk_reduce
+// adds the splits in index order and writes y.
+// It runs with three LDS stages instead of two: its workgroups stream weights that nobody else reads,
+// and two tiles in flight per CU rather than one is what keeps enough bytes on their way from HBM.
+template <int MB, int NB, int WN, bool SPLITK = false>
 __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
     const f16* __restrict__ x, const f16* __restrict__ w, const int64_t* __restrict__ group_list,
-    f16* __restrict__ y, int64_t rows, int k, int num_experts, int n) {
+    f16* __restrict__ y, int64_t rows, int k, int num_experts, int n, float* __restrict__ partial,
+    int splits) {
   constexpr int kWaves = 2 * WN;  // 2 wave rows x WN wave columns
   constexpr int BM = 64 * MB;
   constexpr int BN = 32 * NB * WN;
@@ -270,14 +336,34 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
   constexpr int kBCopies = BN / 8 / kWaves;
   static_assert(BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0, "tile rows per copy");
 
+  constexpr int NS = SPLITK ? 3 : 2;  // LDS stages
   extern __shared__ __attribute__((aligned(16))) f16 smem[];
-  f16* sa = smem;                 // [2][BM * kBK]
-  f16* sb = smem + 2 * BM * kBK;  // [2][BN * kBK]
+  f16* sa = smem;                  // [NS][BM * kBK]
+  f16* sb = smem + NS * BM * kBK;  // [NS][BN * kBK]
 
   const int n_tiles = (n + BN - 1) / BN;
-  const GmmWork work =
-      gmm_find_work<BM>(group_list, num_experts, rows, n_tiles, blockIdx.x, gridDim.x);
-  if (!work.valid) return;
+  GmmWork work;
+  int k_begin = 0;         // first k element of this workgroup's share
+  int ktiles = k / kBK;    // k tiles of this workgroup's share
+  int64_t partial_block = 0;  // SPLITK: index of this workgroup's block of partial results
+  if constexpr (SPLITK) {
+    const int m_tiles = (int)((rows + BM - 1) / BM);
+    const int tile = blockIdx.x / splits;
+    const int split = blockIdx.x - tile * splits;
+    if (tile >= m_tiles * n_tiles) return;
+    partial_block = (int64_t)split * (m_tiles * n_tiles) + tile;
+    work.valid = true;
+    work.expert = 0;
+    work.n_tile = tile / m_tiles;  // the m tiles of one weight tile are adjacent
+    work.row_begin = (tile - work.n_tile * m_tiles) * BM;
+    work.row_end = (int)rows;
+    const int per = (ktiles + splits - 1) / splits;  // the host chooses splits so that none is empty
+    k_begin = split * per * kBK;
+    ktiles = min(per, ktiles - split * per);
+  } else {
+    work = gmm_find_work<BM>(group_list, num_experts, rows, n_tiles, blockIdx.x, gridDim.x);
+    if (!work.valid) return;
+  }
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -293,8 +379,8 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
   // and chunk lane_c: one per-lane offset plus a uniform stride per copy, clamped to the last valid
   // row (tile rows past the end of the group - only dead output rows depend on them - and past
   // the end of w repeat the last valid row).
-  const f16* a_base = x + (int64_t)work.row_begin * k;
-  const f16* b_base = w + ((int64_t)work.expert * n + (int64_t)work.n_tile * BN) * k;
+  const f16* a_base = x + (int64_t)work.row_begin * k + k_begin;
+  const f16* b_base = w + ((int64_t)work.expert * n + (int64_t)work.n_tile * BN) * k + k_begin;
   const int n_left = min(n - work.n_tile * BN, BN);
   const int lane_row = wave * 8 + ((lane >> 3) ^ (wave & 1));
   const int lane_c = (lane & 7) ^ (lane_row & 7);
@@ -302,7 +388,6 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
   const uint32_t copy_stride = 8u * kWaves * (uint32_t)k;
   const uint32_t a_last = (uint32_t)(tile_rows - 1) * (uint32_t)k + lane_c * 8;
   const uint32_t b_last = (uint32_t)(n_left - 1) * (uint32_t)k + lane_c * 8;
-  const int ktiles = k / kBK;
   auto copy_tile = [&](int kt, int stage) {
     const int ko = min(kt, ktiles - 1) * kBK;
     f16* da = sa + stage * BM * kBK + wave * 512;
@@ -363,8 +448,8 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
       if (ST + 1 < kSteps) {
         load_frags((ST + 1) & 1, ST + 1, STAGE);
       } else {
-        load_frags(0, 0, STAGE ^ 1);  // first fragments of the next tile
-        copy_tile(kt + 2, STAGE);     // this stage is free: everyone is past the barrier
+        load_frags(0, 0, (STAGE + 1) % NS);  // first fragments of the next tile
+        copy_tile(kt + NS, STAGE);           // this stage is free: everyone is past the barrier
       }
 #pragma unroll
       for (int i = 0; i < LIVE; ++i)
@@ -380,8 +465,9 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
       step(kt, stage_c, std::integral_constant<int, 0>{});
       step(kt, stage_c, std::integral_constant<int, 1>{});
       step(kt, stage_c, std::integral_constant<int, 2>{});
-      // own copies of tile kt+1 and all own fragment reads of tile kt are complete ...
-      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
+      // own copies of tile kt+1 (later tiles may still be on their way) and all own fragment
+      // reads of tile kt are complete ...
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 2) * (kACopies + kBCopies)));
       asm volatile("" ::: "memory");
       __builtin_amdgcn_s_barrier();  // ... and so are everybody else's
       asm volatile("" ::: "memory");
@@ -390,22 +476,35 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
     };
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
-    // tile 0 must be complete, tile 1 may still be on its way
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kACopies + kBCopies));
+    using I2 = std::integral_constant<int, 2>;
+    // tile 0 must be complete, the later ones may still be on their way
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0((NS - 1) * (kACopies + kBCopies)));
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     load_frags(0, 0, 0);
     int kt = 0;
-    for (; kt + 1 < ktiles; kt += 2) {
-      iteration(kt, I0{});
-      iteration(kt + 1, I1{});
+    if constexpr (NS == 3) {
+      for (; kt + 2 < ktiles; kt += 3) {
+        iteration(kt, I0{});
+        iteration(kt + 1, I1{});
+        iteration(kt + 2, I2{});
+      }
+      if (kt < ktiles) iteration(kt, I0{});
+      if (kt + 1 < ktiles) iteration(kt + 1, I1{});
+    } else {
+      for (; kt + 1 < ktiles; kt += 2) {
+        iteration(kt, I0{});
+        iteration(kt + 1, I1{});
+      }
+      if (kt < ktiles) iteration(kt, I0{});
     }
-    if (kt < ktiles) iteration(kt, I0{});
   };
 
+  static_assert((NS - 1) * (kACopies + kBCopies) < 64, "vmcnt range");
   copy_tile(0, 0);
   copy_tile(1, 1);
+  if constexpr (NS == 3) copy_tile(2, 2);
   if (live >= MB) {
     k_loop(std::integral_constant<int, MB>{});
   } else if (MB > 1 && live == MB - 1) {
@@ -420,45 +519,28 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
 
   // Epilogue: as in grouped_matmul_kernel, one pass per pair of wave columns (BM x 64*NB halfs fit
   // the stages).  The last copies (a repeat of the last tile) must have landed before the stages
-  // are reused for the output tile.
+  // are reused for the output tile (or released).
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
-  __syncthreads();
-  f16* sc = smem;
-  constexpr int kPassCols = 64 * NB;  // columns of two wave columns
-  constexpr int kSwz = (kPassCols / 8 < 16 ? kPassCols / 8 : 16) - 1;
-  constexpr int kChunksPerRow = kPassCols / 8;
-  constexpr int kRowsPerStorePass = kThreads / kChunksPerRow;
+  if constexpr (SPLITK) {
+    f32x4* dst = reinterpret_cast<f32x4*>(partial) + (partial_block * kWaves + wave) * (MB * NB * 4 * kWave) + lane;
 #pragma unroll
-  for (int pass = 0; pass < WN / 2; ++pass) {
-    if (wn / 2 == pass) {
+    for (int i = 0; i < MB; ++i) {
+      if (i < live) {  // the reduction skips the same blocks
 #pragma unroll
-      for (int i = 0; i < MB; ++i) {
-        const int m = 32 * (wm + 2 * i) + fm;
-#pragma unroll
-        for (int j = 0; j < NB; ++j) {
+        for (int j = 0; j < NB; ++j)
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            f16x4 v;
+            f32x4 v;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = (f16)acc[i][j][4 * g + e];
-            const int piece = ((wn & 1) * 32 * NB + 32 * j + 8 * g + 4 * fq) >> 2;
-            *reinterpret_cast<f16x4*>(&sc[m * kPassCols + ((piece ^ ((m & kSwz) << 1)) << 2)]) = v;
+            for (int e = 0; e < 4; ++e) v[e] = acc[i][j][4 * g + e];
+            dst[((i * NB + j) * 4 + g) * kWave] = v;
           }
-        }
       }
     }
-    __syncthreads();
-    const int c16 = tid % kChunksPerRow;
-    const int col = work.n_tile * BN + pass * kPassCols + c16 * 8;
-    if (col < n) {
-      for (int m = tid / kChunksPerRow; m < tile_rows; m += kRowsPerStorePass) {
-        const f16x8 v =
-            *reinterpret_cast<const f16x8*>(&sc[m * kPassCols + ((c16 ^ (m & kSwz)) << 3)]);
-        st128(y + (int64_t)(work.row_begin + m) * n + col, v);
-      }
-    }
-    if (pass + 1 < WN / 2) __syncthreads();
+    return;
   }
+  __syncthreads();
+  gmm_store_tile<MB, NB, WN>(acc, smem, y, work.row_begin, tile_rows, work.n_tile, n);
 }
 
 template <int MB, int NB, int WN>
@@ -484,7 +566,166 @@ static int gmm_dma_launch(const f16* x, const f16* w, const int64_t* group_list,
     attr_set = true;
   }
   kernel<<<(unsigned)grid, 2 * WN * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts,
-                                                          n);
+                                                          n, nullptr, 1);
+  return record_launch_status(hipGetLastError());
+}
+
+// Second kernel of the split-k dense matmul: one wave per (output tile, wave of the first kernel,
+// 64-row block i) adds that block's partial results over the splits, in index order (the result
+// does not depend on which split finished first), and writes it as fp16 straight from registers:
+// lane pairs exchange halves with v_permlane32_swap so that every lane stores 16 contiguous bytes.
+// No LDS, no barrier; the loads of all splits are independent.
+template <int MB, int NB, int WN>
+__global__ __launch_bounds__(4 * kWave) void matmul_splitk_reduce(
+    const float* __restrict__ partial, f16* __restrict__ y, int64_t rows, int n, int splits) {
+  constexpr int kWaves = 2 * WN;
+  constexpr int BM = 64 * MB;
+  constexpr int BN = 32 * NB * WN;
+  const int n_tiles = (n + BN - 1) / BN;
+  const int m_tiles = (int)((rows + BM - 1) / BM);
+  const int tiles = m_tiles * n_tiles;
+  const int unit = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // (tile, wave, i)
+  if (unit >= tiles * kWaves * MB) return;
+  const int i = unit % MB;
+  const int wave = (unit / MB) % kWaves;
+  const int tile = unit / (MB * kWaves);
+  const int n_tile = tile / m_tiles;
+  const int row_begin = (tile - n_tile * m_tiles) * BM;
+  const int tile_rows = min((int)rows - row_begin, BM);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wm = wave / WN;
+  const int wn = wave % WN;
+  const int live = ((tile_rows + 31) / 32 - wm + 1) / 2;
+  if (i >= live) return;  // the first kernel wrote nothing for this block
+  const int fm = lane & 31;
+  const int fq = lane >> 5;
+  f32x4 acc[NB][4];
+#pragma unroll
+  for (int j = 0; j < NB; ++j)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) acc[j][g] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int64_t split_stride = (int64_t)tiles * kWaves * (MB * NB * 4 * kWave);  // float4 units
+  const f32x4* src = reinterpret_cast<const f32x4*>(partial) +
+                     ((int64_t)tile * kWaves + wave) * (MB * NB * 4 * kWave) + (i * NB * 4) * kWave + lane;
+  for (int s = 0; s < splits; ++s) {
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 v = __builtin_nontemporal_load(&src[(j * 4 + g) * kWave]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[j][g][e] += v[e];
+      }
+    src += split_stride;
+  }
+  // acc[j][g][e]: row 32*(wm + 2i) + fm, column wn*32*NB + 32j + 8g + 4fq + e of the tile
+  const int m = 32 * (wm + 2 * i) + fm;
+  const int col_w = n_tile * BN + wn * 32 * NB;
+  const bool row_ok = m < tile_rows;
+  f16* yrow = y + (int64_t)(row_begin + m) * n + col_w + 8 * fq;
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    if (col_w + 32 * j < n) {  // wave uniform: both lanes of every pair take part in the exchange
+#pragma unroll
+      for (int gp = 0; gp < 2; ++gp) {
+        f16x4 p0, p1;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          p0[e] = (f16)acc[j][2 * gp][e];
+          p1[e] = (f16)acc[j][2 * gp + 1][e];
+        }
+        const u32x2 d0 = __builtin_bit_cast(u32x2, p0);
+        const u32x2 d1 = __builtin_bit_cast(u32x2, p1);
+        const auto lo = __builtin_amdgcn_permlane32_swap(d0[0], d1[0], false, false);
+        const auto hi = __builtin_amdgcn_permlane32_swap(d0[1], d1[1], false, false);
+        u32x4 out;
+        out[0] = lo[0];
+        out[1] = hi[0];
+        out[2] = lo[1];
+        out[3] = hi[1];
+        if (row_ok) st128(yrow + 32 * j + 16 * gp, __builtin_bit_cast(f16x8, out));
+      }
+    }
+  }
+}
+
+// Number of k splits worth taking for a dense [m, k] x [n, k]^T product on a device with `cus`
+// CUs: as many as it takes to give every CU a workgroup when the output has too few tiles for
+// that, each split keeping at least eight k tiles; 1 = do not split.
+template <int MB, int NB, int WN>
+static int matmul_splitk_splits(int64_t m, int64_t k, int64_t n, int cus) {
+  constexpr int BM = 64 * MB;
+  constexpr int BN = 32 * NB * WN;
+  const int64_t tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN);
+  const int64_t ktiles = k / kBK;
+  if (tiles * 2 > cus || ktiles < 16) return 1;
+  int64_t splits = cus / tiles;
+  if (splits > ktiles / 8) splits = ktiles / 8;
+  if (splits > 16) splits = 16;
+  if (splits < 2) return 1;
+  const int64_t per = (ktiles + splits - 1) / splits;
+  return (int)((ktiles + per - 1) / per);  // no empty split
+}
+
+constexpr int kSplitMB = 4, kSplitNB = 2, kSplitWN = 2;  // 256 x 128 tiles, four waves
+
+static int device_cus(int* out) {
+  static int cus[64] = {0};  // per device; benign race: every writer stores the same value
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return record_launch_status(e);
+  if (dev < 0 || dev >= 64) return AOPS_ERR_INVALID_ARGUMENT;
+  if (cus[dev] == 0) {
+    int v = 0;
+    e = hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return record_launch_status(e);
+    cus[dev] = v > 0 ? v : 8;
+  }
+  *out = cus[dev];
+  return AOPS_OK;
+}
+
+size_t gmm_splitk_workspace(int64_t m, int64_t k, int64_t n) {
+  int cus = 0;
+  if (device_cus(&cus) != AOPS_OK) return 0;
+  const int splits = matmul_splitk_splits<kSplitMB, kSplitNB, kSplitWN>(m, k, n, cus);
+  if (splits < 2) return 0;
+  constexpr int BM = 64 * kSplitMB;
+  constexpr int BN = 32 * kSplitNB * kSplitWN;
+  const int64_t tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN);
+  return (size_t)splits * (size_t)tiles * BM * BN * sizeof(float);
+}
+
+int gmm_launch_splitk(const f16* x, const f16* w, f16* y, float* workspace, size_t workspace_bytes,
+                      int64_t m, int k, int n, hipStream_t stream) {
+  constexpr int MB = kSplitMB, NB = kSplitNB, WN = kSplitWN;
+  constexpr int BM = 64 * MB;
+  constexpr int BN = 32 * NB * WN;
+  int cus = 0;
+  const int rc = device_cus(&cus);
+  if (rc != AOPS_OK) return rc;
+  const int splits = matmul_splitk_splits<MB, NB, WN>(m, k, n, cus);
+  const int64_t tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN);
+  if (splits < 2) return AOPS_ERR_INVALID_ARGUMENT;
+  if (!workspace || workspace_bytes < (size_t)splits * (size_t)tiles * BM * BN * sizeof(float))
+    return AOPS_ERR_WORKSPACE;
+  constexpr int kStageBytes = 3 * (BM + BN) * kBK * (int)sizeof(f16);
+  static_assert(kStageBytes <= 160 * 1024, "LDS budget");
+  auto kernel = grouped_matmul_dma_kernel<MB, NB, WN, true>;
+  auto reduce = matmul_splitk_reduce<MB, NB, WN>;
+  static bool attr_set = false;  // benign race: the calls are idempotent
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes);
+    if (e != hipSuccess) return record_launch_status(e);
+    attr_set = true;
+  }
+  kernel<<<(unsigned)(tiles * splits), 2 * WN * kWave, kStageBytes, stream>>>(x, w, nullptr, y, m, k, 1, n,
+                                                                            workspace, splits);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return record_launch_status(e);
+  const int64_t units = tiles * (2 * WN) * MB;  // one wave each
+  reduce<<<(unsigned)((units + 3) / 4), 4 * kWave, 0, stream>>>(workspace, y, m, n, splits);
   return record_launch_status(hipGetLastError());
 }
 

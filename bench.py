@@ -288,11 +288,22 @@ def _gmm_entry(L, ops, R, dev, cpu, op, config, x, w_storage, gl, note=None, che
     ws = [wd] + [wd.clone() for _ in range(n - 1)]
     ys = [torch.empty(rows, N, dtype=torch.float16, device=dev) for _ in range(n)]
 
+    # what ops.grouped_matmul does: one expert with few rows and a long k goes to the dense split-k entry point
+    ws_bytes = L.lib.aops_matmul_nt_workspace(rows, K, N) if E == 1 else 0
+    scratch = [torch.empty(ws_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] if ws_bytes else None
+
     def mk(i):
+        if ws_bytes:
+            return lambda: L.check(L.lib.aops_matmul_nt_ws_f16(xs[i].data_ptr(), ws[i].data_ptr(), ys[i].data_ptr(),
+                                                               scratch[i].data_ptr(), ws_bytes, rows, K, N, L.stream()))
         return lambda: L.check(L.lib.aops_grouped_matmul_f16(xs[i].data_ptr(), ws[i].data_ptr(), gd.data_ptr(),
                                                             ys[i].data_ptr(), rows, K, E, N, L.stream()))
 
     med, mn = time_graph([mk(i) for i in range(n)], min_launches=40)
+    if ws_bytes:
+        note = (note + "; " if note else "") + (
+            f"two kernels per call: k range split over the workgroups of a tile ({ws_bytes / 1e6:.1f} MB of fp32 "
+            "partial results) + reduction")
     eager = time_eager([(lambda i=i: ops.grouped_matmul(xs[i], ws[i].transpose(1, 2), gd)) for i in range(n)], 3, 20)
     w_logical = w_storage.transpose(1, 2)
     cpu_ms = None

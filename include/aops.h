@@ -147,6 +147,23 @@ int aops_matmul_nt_f16(const void* x, const void* w, void* y, int64_t m, int64_t
                        void* stream);
 
 /*
+ * The same product for shapes with few rows and a long k (a decode-time down projection:
+ * 256 x 14336 -> 4096), where whole-k output tiles would leave most CUs idle: the k range is
+ * split over several workgroups per tile, the fp32 partial results go to `workspace` and a second
+ * kernel adds them in a fixed order (deterministic) and writes y.
+ * aops_matmul_nt_workspace returns the bytes of device scratch the call needs on the current
+ * device, or 0 when splitting does not pay for the shape; aops_matmul_nt_ws_f16 then computes
+ * exactly what aops_matmul_nt_f16 does and ignores the workspace.  A workspace that is required
+ * but missing or too small returns AOPS_ERR_WORKSPACE.  The workspace may be freed or reused as
+ * soon as the call's work on `stream` is done; calls on different streams need their own.
+ * Same reference counterpart as aops_matmul_nt_f16 (the reference's two-phase
+ * GetWorkspaceSize + launch convention, reference csrc/ffi/ops.cpp:211-218, kept visible).
+ */
+size_t aops_matmul_nt_workspace(int64_t m, int64_t k, int64_t n);
+int aops_matmul_nt_ws_f16(const void* x, const void* w, void* y, void* workspace,
+                          size_t workspace_bytes, int64_t m, int64_t k, int64_t n, void* stream);
+
+/*
  * Grouped matmul of a gate_up projection with the SwiGLU activation fused into its epilogue:
  *   h = x[rows of expert e] (fp32 accumulate) @ w[e]^T          (never stored)
  *   y[r, c] = f16( silu(h[r, c]) * h[r, n/2 + c] ),  c < n/2

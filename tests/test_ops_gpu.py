@@ -374,6 +374,57 @@ def test_matmul_nt(ops, dev, m, k, n):
     torch.testing.assert_close(y.cpu().float(), x.float() @ w.float().T, **GMM_TOL)
 
 
+SPLIT_K_SHAPES = [(256, 14336, 4096), (16, 8192, 1024), (300, 4096, 256), (1, 2048, 64), (257, 64 * 37, 192),
+                  (64, 1024, 2048), (512, 16384, 128)]
+
+
+@pytest.mark.parametrize("m,k,n", SPLIT_K_SHAPES)
+def test_matmul_nt_split_k(ops, dev, m, k, n):
+    """Few rows and a long k: the k range is split over workgroups and a second kernel adds the partial results.
+    Against the fp32 product, against the whole-k kernels, and bit-identical from call to call."""
+    import ascend910a_extras.ascend910a_extras_C as C
+
+    g = _gen(m + k + n)
+    x = torch.randn(m, k, generator=g).half()
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).half()
+    xd, wd = x.to(dev), w.to(dev)
+    ws_bytes = C._lib.aops_matmul_nt_workspace(m, k, n)
+    assert ws_bytes > 0, "the shape is meant to take the split-k path"
+    y = ops.matmul(xd, wd)
+    ref = x.float() @ w.float().T
+    torch.testing.assert_close(y.cpu().float(), ref, **GMM_TOL)
+    # the whole-k kernel (no workspace) agrees to rounding: both accumulate in fp32, in a different order
+    whole = torch.empty_like(y)
+    assert C._lib.aops_matmul_nt_f16(xd.data_ptr(), wd.data_ptr(), whole.data_ptr(), m, k, n, C._stream(dev)) == 0
+    torch.testing.assert_close(y.float(), whole.float(), rtol=2e-3, atol=2e-3)
+    assert torch.equal(ops.matmul(xd, wd), y)
+    # one expert through the grouped entry of the Python API takes the same path
+    gl = torch.tensor([m], dtype=torch.int64, device=dev)
+    assert torch.equal(ops.grouped_matmul(xd, wd[None].transpose(1, 2), gl), y)
+    # a workspace that is too small is refused, the output untouched
+    small = torch.empty(ws_bytes - 1, dtype=torch.uint8, device=dev)
+    out = torch.zeros_like(y)
+    code = C._lib.aops_matmul_nt_ws_f16(xd.data_ptr(), wd.data_ptr(), out.data_ptr(), small.data_ptr(), ws_bytes - 1,
+                                        m, k, n, C._stream(dev))
+    torch.cuda.synchronize()
+    assert code == -2 and not out.any()
+
+
+def test_matmul_nt_ws_without_split(ops, dev):
+    """Shapes with enough output tiles need no workspace; the workspace entry point then equals the plain one."""
+    import ascend910a_extras.ascend910a_extras_C as C
+
+    m, k, n = 512, 512, 8192
+    assert C._lib.aops_matmul_nt_workspace(m, k, n) == 0
+    g = _gen(5)
+    x = torch.randn(m, k, generator=g).half().to(dev)
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).half().to(dev)
+    a, b = torch.empty(m, n, dtype=H, device=dev), torch.empty(m, n, dtype=H, device=dev)
+    assert C._lib.aops_matmul_nt_ws_f16(x.data_ptr(), w.data_ptr(), a.data_ptr(), None, 0, m, k, n, C._stream(dev)) == 0
+    assert C._lib.aops_matmul_nt_f16(x.data_ptr(), w.data_ptr(), b.data_ptr(), m, k, n, C._stream(dev)) == 0
+    assert torch.equal(a, b)
+
+
 def test_dense_mlp_chain(ops, dev):
     """benchmark/test_mlp.py:37-41 through grouped_matmul with one expert (reduced width)."""
     g = _gen(0)
