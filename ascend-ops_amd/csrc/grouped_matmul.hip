@@ -35,19 +35,36 @@ static int aops_grouped_matmul_impl(const void* x, const void* w, const int64_t*
   const f16* xp = static_cast<const f16*>(x);
   const f16* wp = static_cast<const f16*>(w);
   f16* yp = static_cast<f16*>(y);
-  const char* forced_env = getenv("AOPS_GMM_VARIANT");  // tuning aid: 1..8 force one kernel / tile shape
+  const char* forced_env = getenv("AOPS_GMM_VARIANT");  // tuning aid: 1..9 force one kernel / tile shape
   const int forced = forced_env ? atoi(forced_env) : 0;
-  // Tile choice from what the host knows (group_list stays on the device): the largest tile
-  // whose grid still gives every CU work.  320 rows cover a typical expert of a large routed
-  // batch in one tile; small or dense problems (few rows, one expert) take smaller tiles so that
-  // enough workgroups exist to pull the weights through all memory channels.
+  // Tile choice from what the host knows (group_list stays on the device, so the rows are taken
+  // to be spread evenly over the experts).  With few rows per expert the weights are streamed for
+  // little arithmetic and every tile row beyond the group is wasted copy and MFMA work: 128- or
+  // 64-row tiles.  Otherwise the largest tile whose grid still gives most CUs a work item: 320
+  // rows cover a typical expert of a large routed batch in one tile, and the persistent kernel
+  // (320 x 256) wins as soon as there are enough items for one per CU.
   int variant = forced;
-  if (variant < 1 || variant > 8) {
-    auto tiles = [&](int64_t bm, int64_t bn) { return ((rows + bm - 1) / bm) * ((n + bn - 1) / bn); };
-    constexpr int64_t kEnough = 384;
-    constexpr int64_t kMostCus = 192;  // 256-row tiles read a small batch's weights once: worth a few idle CUs
-    variant = tiles(320, 256) >= kEnough ? 6 : tiles(320, 128) >= kEnough ? 2 : tiles(256, 128) >= kMostCus ? 3
-              : tiles(128, 128) >= kEnough ? 4 : 5;
+  if (variant < 1 || variant > 9) {
+    const int64_t groups = num_experts < rows ? num_experts : rows;  // experts that can hold a row
+    const int64_t avg = (rows + groups - 1) / groups;
+    auto m_tiles = [&](int64_t bm) { return (avg + bm - 1) / bm; };
+    auto items = [&](int64_t bm, int64_t bn) { return groups * m_tiles(bm) * ((n + bn - 1) / bn); };
+    constexpr int64_t kEnough = 190;  // of 256 CUs
+    if (avg < 96) {
+      variant = (avg >= 24 && items(128, 128) >= kEnough) ? 4 : 5;
+    } else if (items(320, 256) >= kEnough) {
+      variant = 6;
+    } else if (items(256, 128) >= kEnough && m_tiles(256) * 256 < m_tiles(320) * 320) {
+      variant = 3;  // pads the groups less than 320-row tiles would
+    } else if (items(320, 128) >= kEnough) {
+      variant = 2;
+    } else if (items(256, 128) >= kEnough) {
+      variant = 3;
+    } else if (items(128, 128) >= kEnough) {
+      variant = 4;
+    } else {
+      variant = 5;
+    }
   }
   if (variant == 6 && (k % 128 != 0 || k < 256)) variant = 1;  // the persistent kernel's k loop
   if (variant == 6)  // 320 x 256 tiles, eight waves, one persistent workgroup per CU

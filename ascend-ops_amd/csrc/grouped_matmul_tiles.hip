@@ -322,7 +322,7 @@ __device__ __forceinline__ void gmm_store_tile(const f32x16 (&acc)[MB][NB], f16*
 // adds the splits in index order and writes y.
 // It runs with three LDS stages instead of two: its workgroups stream weights that nobody else reads,
 // and two tiles in flight per CU rather than one is what keeps enough bytes on their way from HBM.
-template <int MB, int NB, int WN, bool SPLITK = false>
+template <int MB, int NB, int WN, bool SPLITK = false, int NS = (SPLITK ? 3 : 2)>
 __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
     const f16* __restrict__ x, const f16* __restrict__ w, const int64_t* __restrict__ group_list,
     f16* __restrict__ y, int64_t rows, int k, int num_experts, int n, float* __restrict__ partial,
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
   constexpr int kBCopies = BN / 8 / kWaves;
   static_assert(BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0, "tile rows per copy");
 
-  constexpr int NS = SPLITK ? 3 : 2;  // LDS stages
+  static_assert(NS == 2 || NS == 3, "LDS stages");
   extern __shared__ __attribute__((aligned(16))) f16 smem[];
   f16* sa = smem;                  // [NS][BM * kBK]
   f16* sb = smem + NS * BM * kBK;  // [NS][BN * kBK]
@@ -543,12 +543,12 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_dma_kernel(
   gmm_store_tile<MB, NB, WN>(acc, smem, y, work.row_begin, tile_rows, work.n_tile, n);
 }
 
-template <int MB, int NB, int WN>
+template <int MB, int NB, int WN, int NS = 2>
 static int gmm_dma_launch(const f16* x, const f16* w, const int64_t* group_list, f16* y,
                           int64_t rows, int k, int num_experts, int n, hipStream_t stream) {
   constexpr int BM = 64 * MB;
   constexpr int BN = 32 * NB * WN;
-  constexpr int kStageBytes = 2 * (BM + BN) * kBK * (int)sizeof(f16);
+  constexpr int kStageBytes = NS * (BM + BN) * kBK * (int)sizeof(f16);
   constexpr int kTileBytes = BM * 64 * NB * (int)sizeof(f16);
   constexpr int kLds = kStageBytes > kTileBytes ? kStageBytes : kTileBytes;
   static_assert(kLds <= 160 * 1024, "LDS budget");
@@ -557,7 +557,7 @@ static int gmm_dma_launch(const f16* x, const f16* w, const int64_t* group_list,
   int64_t grid = max_m_tiles * n_tiles;
   grid = (grid + kXcds - 1) / kXcds * kXcds;
   if (grid > 0x7fffffff) return AOPS_ERR_INVALID_ARGUMENT;
-  auto kernel = grouped_matmul_dma_kernel<MB, NB, WN>;
+  auto kernel = grouped_matmul_dma_kernel<MB, NB, WN, false, NS>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -764,6 +764,8 @@ int gmm_launch_tiles(int variant, const f16* x, const f16* w, const int64_t* gro
       return gmm_dma_launch<4, 2, 2>(x, w, group_list, y, rows, k, num_experts, n, stream);
     case 8:  // 128 x 128 tiles, four waves, operands copied HBM -> LDS directly
       return gmm_dma_launch<2, 2, 2>(x, w, group_list, y, rows, k, num_experts, n, stream);
+    case 9:  // 256 x 128 tiles, four waves, three LDS stages
+      return gmm_dma_launch<4, 2, 2, 3>(x, w, group_list, y, rows, k, num_experts, n, stream);
     case 2:  // 320 x 128 tiles
       return gmm_launch<5, 2, 2>(x, w, group_list, y, rows, k, num_experts, n, stream);
     case 3:  // 256 x 128 tiles

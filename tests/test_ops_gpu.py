@@ -306,7 +306,7 @@ def test_grouped_matmul_does_not_write_past_the_last_group(ops, dev):
     torch.testing.assert_close(y.cpu()[:110].float(), ref[:110].float(), **GMM_TOL)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9])
 @pytest.mark.parametrize(
     "rows,K,N,E,counts",
     [
