@@ -23,7 +23,8 @@
 //    [token][16 d] blocks whose result layout has 4 consecutive tokens per lane; converted
 //    back to fp16 (exact) they are the V^T operand.
 //  * The K registers are refilled for the next step as soon as the scores are out, the V
-//    registers as soon as P.V is done; three workgroups per CU cover each other's waits.
+//    registers as soon as P.V is done; the eight waves of the one workgroup a CU holds cover
+//    each other's waits.
 //
 // Semantics: signature, cache indexing, GQA mapping and the fixed 1/sqrt(D) scale follow
 // reference csrc/ffi/ops.cpp:408-482, csrc/opdev/op_host/paged_attention_ex.cpp:18-36 and
@@ -59,7 +60,7 @@ static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_si
   int chunk = (int)(((max_units + splits - 1) / splits) * kUnit);
   if (chunk < kUnit) chunk = kUnit;
   static const int forced = [] {
-    const char* e = getenv("AOPS_PA_CHUNK");  // tuning aid; must be a multiple of 128
+    const char* e = getenv("AOPS_PA_CHUNK");  // tuning aid; a multiple of 256 tokens, ignored otherwise
     const int v = e ? atoi(e) : 0;
     return (v >= kPaWaves * kPaStep && v % (kPaWaves * kPaStep) == 0) ? v : 0;
   }();
@@ -160,7 +161,7 @@ __device__ __forceinline__ void pa_accumulate(const PaRegs& v, const f16x8 (&sel
   }
 }
 
-// grid = (max_splits, Hkv, bs), block = 256.  G = query heads per kv head (<= 16).
+// grid = (max_splits, Hkv, bs), block = 8 waves.  G = query heads per kv head (<= 16).
 // FINAL: the chunk is the whole sequence, so the normalised output is written directly.
 template <int G, bool FINAL>
 __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
