@@ -620,3 +620,73 @@ def test_print_info(ops, dev, capsys):
     ops.print_info()
     out = capsys.readouterr().out
     assert "compute units" in out and "gfx" in out
+
+
+def test_caches_larger_than_4_gib(ops, dev):
+    """Page offsets beyond 2^32 bytes (and 2^31 elements): reshape_and_cache, the fused rope + cache write and paged
+    attention on 5.4 GB caches whose pages in use lie at the far end.  Only those pages are ever initialised or
+    copied to the host; the oracle works on a compact copy with a remapped block table."""
+    import ascend910a_extras.fused as fused
+
+    g = _gen(77)
+    NB, Hkv, Hq, D, P = 20480, 8, 32, 128, 128
+    assert NB * (Hkv * D // 16) * P * 16 > 2 ** 31
+    kc = torch.empty(NB, Hkv * D // 16, P, 16, dtype=H, device=dev)
+    vc = torch.empty_like(kc)
+    B, lens = 3, [300, 128, 1]
+    used = [NB - 1, NB - 7, 16400, NB - 300, 17000]                 # pages beyond element 2^31, not in order
+    bt = torch.tensor([[used[0], used[1], used[2]], [used[3], 0, 0], [used[4], 0, 0]], dtype=torch.int32)
+    small_k = torch.randn(len(used), Hkv * D // 16, P, 16, generator=g).half()
+    small_v = torch.randn(len(used), Hkv * D // 16, P, 16, generator=g).half()
+    idx = torch.tensor(used, device=dev)
+    kc[idx] = small_k.to(dev)
+    vc[idx] = small_v.to(dev)
+    remap = {p: i for i, p in enumerate(used)}
+    bt_small = torch.tensor([[remap.get(int(p), 0) for p in row] for row in bt], dtype=torch.int32)
+    cl = torch.tensor(lens, dtype=torch.int32)
+    # the newest token of every sequence arrives through rope + cache write
+    q = torch.randn(B, Hq, D, generator=g).half()
+    k = torch.randn(B, Hkv, D, generator=g).half()
+    v = torch.randn(B, Hkv, D, generator=g).half()
+    pos = (cl - 1).int()
+    cos, sin = R.build_cos_sin_cache(512, D)
+    slots = torch.tensor([int(bt[b, int(pos[b]) // P]) * P + int(pos[b]) % P for b in range(B)], dtype=torch.int32)
+    slots_small = torch.tensor([int(bt_small[b, int(pos[b]) // P]) * P + int(pos[b]) % P for b in range(B)], dtype=torch.int32)
+    assert int(slots.max()) * (Hkv * D) > 2 ** 31
+    oq = fused.rope_reshape_and_cache(q.to(dev), k.to(dev), v.to(dev), pos.to(dev), cos.to(dev), sin.to(dev), kc, vc,
+                                      slots.to(dev))
+    rq, rk = R.rope_ref(q, k, pos, cos, sin)
+    R.reshape_and_cache_ref(rk, small_k, slots_small, v, small_v)
+    assert torch.equal(kc[idx].cpu(), small_k) and torch.equal(vc[idx].cpu(), small_v)
+    # the plain operator writes the same bytes
+    kc2 = torch.empty_like(kc)
+    ops.reshape_and_cache(rk.to(dev), None, kc2, None, slots.to(dev))
+    for b in range(B):
+        page, off = int(slots[b]) // P, int(slots[b]) % P
+        assert torch.equal(kc2[page, :, off, :].cpu(), small_k[remap[page], :, off, :])
+    del kc2
+    o = ops.paged_attention(oq, kc, vc, bt.to(dev), cl.to(dev)).cpu()
+    ref = R.paged_attention_ref(rq, small_k, small_v, bt_small, cl)
+    torch.testing.assert_close(o.float(), ref.float(), **TOL)
+
+
+def test_grouped_matmul_more_than_2_31_elements(ops, dev):
+    """Row offsets beyond 2^31 elements of x (4.9 GB of activations): slices at the start, across a group boundary far
+    into the matrix and at the very end against the fp32 product of the same rows."""
+    rows, K, N, E = 1_200_000, 2048, 64, 3
+    assert rows * K > 2 ** 31
+    g = torch.Generator(device=dev).manual_seed(5)
+    x = torch.empty(rows, K, dtype=H, device=dev)
+    for r0 in range(0, rows, 100_000):
+        x[r0:r0 + 100_000] = torch.randn(min(100_000, rows - r0), K, generator=g, device=dev).half()
+    w = (torch.randn(E, N, K, generator=g, device=dev) / K ** 0.5).half().transpose(1, 2)
+    bounds = [400_000, 800_037, rows]
+    gl = torch.tensor(bounds, dtype=torch.int64, device=dev)
+    y = ops.grouped_matmul(x, w, gl)
+    for lo, hi in ((0, 512), (800_037 - 300, 800_037 + 300), (rows - 512, rows)):
+        xs = x[lo:hi].float().cpu()
+        ref = torch.empty(hi - lo, N)
+        for r in range(lo, hi):
+            e = sum(r >= b for b in bounds)
+            ref[r - lo] = xs[r - lo] @ w[e].float().cpu()
+        torch.testing.assert_close(y[lo:hi].cpu().float(), ref, **GMM_TOL)
