@@ -8,7 +8,8 @@
 // read on the device only, so the grid is sized for the longest possible context and
 // workgroups past the end of their sequence exit at once.
 //
-// Main kernel (head_dim 128), one step = 32 tokens of one kv head = 8 KiB of K + 8 KiB of V:
+// Main kernel (head_dim 64, 128 or 256; described for 128), one step = 32 tokens of one kv head =
+// 8 KiB of K + 8 KiB of V:
 //  * For one kv head a page holds K as [8 d-chunks][block_size tokens][16 halfs].  A lane
 //    (n = lane%16, kg = lane/16) loads, for token n of a 16-token group, the 16 bytes that hold
 //    d = 32s + 8kg ..+7 (s = 0..3).  That register IS the per-lane operand of
@@ -35,7 +36,6 @@
 
 namespace aops {
 
-constexpr int kPaD = 128;     // head_dim of the fast path
 constexpr int kPaWaves = 8;   // waves per workgroup
 constexpr int kPaStep = 32;   // tokens per wave per step (two 16-token MFMA groups)
 constexpr float kNegBig = -1.0e30f;
@@ -72,33 +72,40 @@ static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_si
   return c;
 }
 
-// Per-lane slice of a 32-token tile: [token group][s] holds X[token 16t + n][d = 32s + 8kg ..+7].
-typedef f16x8 PaRegs[2][4];
+// Per-lane slice of a 32-token tile: [token group][s] holds X[token 16t + n][d = 32s + 8kg ..+7],
+// s = 0 .. NS-1 with NS = head_dim / 32.
+template <int NS>
+using PaRegs = f16x8[2][NS];
 
-__device__ __forceinline__ void pa_issue_loads(const f16* __restrict__ base, uint32_t lane_off,
-                                               uint32_t s_stride, PaRegs& r) {
+template <int NS>
+__device__ __forceinline__ void pa_issue_loads(const f16* __restrict__ cache, int64_t off0, int64_t off1,
+                                               uint32_t lane_off, uint32_t s_stride, PaRegs<NS>& r) {
 #pragma unroll
-  for (int g = 0; g < 2; ++g)
+  for (int g = 0; g < 2; ++g) {
+    const f16* base = cache + (g == 0 ? off0 : off1) + lane_off;  // token group g of the step
 #pragma unroll
-    for (int s = 0; s < 4; ++s) r[g][s] = ld128_stream(base + lane_off + s * s_stride + g * 256);
+    for (int s = 0; s < NS; ++s) r[g][s] = ld128_stream(base + s * s_stride);
+  }
 }
 
+template <int NS>
 struct PaState {
-  f32x4 o[8];  // O^T blocks: lane (head n, kg), o[db][i] <-> d = 16 db + 4 kg + i
+  f32x4 o[2 * NS];  // O^T blocks: lane (head n, kg), o[db][i] <-> d = 16 db + 4 kg + i
   float m;     // running maximum of head n (identical in the four lanes of a head)
   float l;     // this lane's share of the running sum
 };
 
 // S^T[token][head] = K . Q^T, scaled to log2 units; lane (head n, kg) gets tokens
 // 16*(e/4) + 4kg + e%4, e = 0..7, of the step.
-__device__ __forceinline__ void pa_scores(const PaRegs& k, const f16x8 (&qreg)[4],
+template <int NS>
+__device__ __forceinline__ void pa_scores(const PaRegs<NS>& k, const f16x8 (&qreg)[NS],
                                           float scale_log2, float (&sc)[8]) {
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
   f32x4 sacc[2] = {zero4, zero4};
 #pragma unroll
   for (int g = 0; g < 2; ++g)
 #pragma unroll
-    for (int s = 0; s < 4; ++s)
+    for (int s = 0; s < NS; ++s)
       sacc[g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(k[g][s], qreg[s], sacc[g], 0, 0, 0);
   // A matrix-core result may only be read six wait states after its instruction (four passes plus
   // two).  The compiler keeps that distance inside a basic block, but when it places the
@@ -114,7 +121,8 @@ __device__ __forceinline__ void pa_scores(const PaRegs& k, const f16x8 (&qreg)[4
 }
 
 // Online softmax update; returns the P^T operand (lane (head n, kg), element e <-> token e).
-__device__ __forceinline__ f16x8 pa_softmax(float (&sc)[8], PaState& st) {
+template <int NS>
+__device__ __forceinline__ f16x8 pa_softmax(float (&sc)[8], PaState<NS>& st) {
   float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
                    fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
   mx = fmaxf(mx, __shfl_xor(mx, 16));
@@ -132,7 +140,7 @@ __device__ __forceinline__ f16x8 pa_softmax(float (&sc)[8], PaState& st) {
   st.l = st.l * alpha + psum;
   if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {  // the maximum rarely moves after the start
 #pragma unroll
-    for (int db = 0; db < 8; ++db)
+    for (int db = 0; db < 2 * NS; ++db)
 #pragma unroll
       for (int i = 0; i < 4; ++i) st.o[db][i] *= alpha;
   }
@@ -140,11 +148,12 @@ __device__ __forceinline__ f16x8 pa_softmax(float (&sc)[8], PaState& st) {
 }
 
 // O^T += V^T . P^T with V transposed on the matrix core.
-__device__ __forceinline__ void pa_accumulate(const PaRegs& v, const f16x8 (&sel)[2], f16x8 pt,
-                                              PaState& st) {
+template <int NS>
+__device__ __forceinline__ void pa_accumulate(const PaRegs<NS>& v, const f16x8 (&sel)[2], f16x8 pt,
+                                              PaState<NS>& st) {
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
+  for (int s = 0; s < NS; ++s) {
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       // [token][d = 32s + 16u + n]: lane (n, kg) receives tokens 4kg..4kg+3 of each group
@@ -161,15 +170,18 @@ __device__ __forceinline__ void pa_accumulate(const PaRegs& v, const f16x8 (&sel
   }
 }
 
-// grid = (max_splits, Hkv, bs), block = 8 waves.  G = query heads per kv head (<= 16).
+// grid = (max_splits, Hkv, bs), block = 8 waves.  `group` = query heads per kv head, GMAX = the
+// power of two it is rounded up to (<= 16; sizes the LDS arrays).
 // FINAL: the chunk is the whole sequence, so the normalised output is written directly.
-template <int G, bool FINAL>
+template <int D, int GMAX, bool FINAL>
 __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
     const f16* __restrict__ q, const f16* __restrict__ key_cache,
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ context_lens, float* __restrict__ part_o,
     float* __restrict__ part_ml, f16* __restrict__ out, int num_kv_heads, int block_size, int max_blocks_per_seq,
-    int chunk_tokens, int max_splits, float scale_log2, int num_blocks) {
+    int chunk_tokens, int max_splits, float scale_log2, int num_blocks, int group) {
+  constexpr int kPaD = D;
+  constexpr int NS = D / 32;
   const int split = blockIdx.x;
   const int g = blockIdx.y;
   // Workgroups are handed out in index order, so they take the sequences longest first: with
@@ -193,8 +205,8 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
   const int chunk_start = split * chunk_tokens;
   if (chunk_start >= context_len) {
     if (FINAL) {  // empty sequence: zeros
-      for (int e = threadIdx.x; e < G * kPaD; e += kPaWaves * kWave)
-        out[((int64_t)b * num_kv_heads * G + g * G) * kPaD + e] = (f16)0.f;
+      for (int e = threadIdx.x; e < group * kPaD; e += kPaWaves * kWave)
+        out[((int64_t)b * num_kv_heads * group + g * group) * kPaD + e] = (f16)0.f;
     }
     return;
   }
@@ -205,15 +217,15 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
   const int lane = threadIdx.x & (kWave - 1);
   const int n = lane & 15;
   const int kg = lane >> 4;
-  const int num_heads = num_kv_heads * G;
+  const int num_heads = num_kv_heads * group;
 
-  // Q^T operand: lane (head n, kg) holds q[head n][32s + 8kg ..+7]; heads >= G are zero rows.
-  f16x8 qreg[4];
+  // Q^T operand: lane (head n, kg) holds q[head n][32s + 8kg ..+7]; heads >= group are zero rows.
+  f16x8 qreg[NS];
   {
     const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    const f16* qp = q + ((int64_t)b * num_heads + g * G + (n < G ? n : 0)) * kPaD + 8 * kg;
+    const f16* qp = q + ((int64_t)b * num_heads + g * group + (n < group ? n : 0)) * kPaD + 8 * kg;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) qreg[s] = n < G ? ld128(qp + 32 * s) : zero8;
+    for (int s = 0; s < NS; ++s) qreg[s] = n < group ? ld128(qp + 32 * s) : zero8;
   }
   // Selector operands of the transposing product: sel[u][k][n] = (k == n + 16u), k = 8kg + e.
   f16x8 sel[2];
@@ -222,9 +234,9 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
 #pragma unroll
     for (int e = 0; e < 8; ++e) sel[u][e] = (8 * kg + e == n + 16 * u) ? (f16)1.0f : (f16)0.0f;
 
-  PaState st;
+  PaState<NS> st;
 #pragma unroll
-  for (int db = 0; db < 8; ++db) st.o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int db = 0; db < 2 * NS; ++db) st.o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
   st.m = kNegBig;
   st.l = 0.f;
 
@@ -237,30 +249,33 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
   const int64_t head_off = (int64_t)g * kPaD * block_size;
   const int32_t* table = block_tables + (int64_t)b * max_blocks_per_seq;
 
-  auto page_offset = [&](int step) -> int64_t {
-    const int tok = chunk_start + step * kPaStep;  // first token of the step (wave uniform)
-    const int blk = tok / block_size;
+  // Offset of the 16-token group `grp` of a step (wave uniform).  Page sizes are multiples of 16, so a
+  // group never straddles two pages; the two groups of a step may (page sizes that are odd multiples).
+  auto page_offset = [&](int step, int grp) -> int64_t {
+    const int tok = chunk_start + step * kPaStep + 16 * grp;
+    const int blk = min(tok / block_size, max_blocks_per_seq - 1);  // the group past the end of the last page
     // a table entry outside the cache reads the nearest page instead of faulting
     const int64_t page = min(max(table[blk], 0), num_blocks - 1);
-    return page * page_elems + head_off + (int64_t)(tok - blk * block_size) * 16;
+    return page * page_elems + head_off + (int64_t)(tok - (tok / block_size) * block_size) * 16;
   };
 
-  PaRegs kreg, vreg;
+  PaRegs<NS> kreg, vreg;
   int step = wave;
   if (step < nsteps) {
-    const int64_t off = page_offset(step);
-    pa_issue_loads(key_cache + off, lane_off, s_stride, kreg);
-    pa_issue_loads(value_cache + off, lane_off, s_stride, vreg);
+    const int64_t off0 = page_offset(step, 0), off1 = page_offset(step, 1);
+    pa_issue_loads(key_cache, off0, off1, lane_off, s_stride, kreg);
+    pa_issue_loads(value_cache, off0, off1, lane_off, s_stride, vreg);
   }
   while (step < nsteps) {
     const int next = step + kPaWaves;
     const bool has_next = next < nsteps;
-    const int64_t next_off = has_next ? page_offset(next) : 0;
+    const int64_t next_off0 = has_next ? page_offset(next, 0) : 0;
+    const int64_t next_off1 = has_next ? page_offset(next, 1) : 0;
     const int step_token0 = chunk_start + step * kPaStep;
     float sc[8];
     pa_scores(kreg, qreg, scale_log2, sc);
     // K registers are free again: the next step's K is in flight during softmax and P.V.
-    if (has_next) pa_issue_loads(key_cache + next_off, lane_off, s_stride, kreg);
+    if (has_next) pa_issue_loads(key_cache, next_off0, next_off1, lane_off, s_stride, kreg);
     if (step_token0 + kPaStep > context_len) {  // wave uniform: last, partial step of the sequence
       // Cache contents past the end of the sequence are arbitrary (possibly NaN): drop their
       // scores and zero their V rows before they reach the matrix core.
@@ -272,13 +287,13 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
           if (step_token0 + 16 * g + 4 * kg + i >= context_len) sc[4 * g + i] = -__builtin_inff();
         if (step_token0 + 16 * g + n >= context_len) {
 #pragma unroll
-          for (int s = 0; s < 4; ++s) vreg[g][s] = zero8;
+          for (int s = 0; s < NS; ++s) vreg[g][s] = zero8;
         }
       }
     }
     const f16x8 pt = pa_softmax(sc, st);
     pa_accumulate(vreg, sel, pt, st);
-    if (has_next) pa_issue_loads(value_cache + next_off, lane_off, s_stride, vreg);
+    if (has_next) pa_issue_loads(value_cache, next_off0, next_off1, lane_off, s_stride, vreg);
     step = next;
   }
 
@@ -288,12 +303,12 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
   l_head += __shfl_xor(l_head, 32);
 
   // Merge the waves of the workgroup through LDS and emit one partial per query head.
-  __shared__ float sm_acc[kPaWaves][G][kPaD];
-  __shared__ float sm_m[kPaWaves][G];
-  __shared__ float sm_l[kPaWaves][G];
-  if (n < G) {
+  __shared__ float sm_acc[kPaWaves][GMAX][kPaD];
+  __shared__ float sm_m[kPaWaves][GMAX];
+  __shared__ float sm_l[kPaWaves][GMAX];
+  if (n < group) {
 #pragma unroll
-    for (int db = 0; db < 8; ++db)
+    for (int db = 0; db < 2 * NS; ++db)
       *reinterpret_cast<f32x4*>(&sm_acc[wave][n][16 * db + 4 * kg]) = st.o[db];
     if (kg == 0) {
       sm_m[wave][n] = st.m;
@@ -301,7 +316,7 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
     }
   }
   __syncthreads();
-  for (int e = threadIdx.x; e < G * kPaD; e += kPaWaves * kWave) {
+  for (int e = threadIdx.x; e < group * kPaD; e += kPaWaves * kWave) {
     const int h = e / kPaD;
     const int d = e - h * kPaD;
     float mx = sm_m[0][h];
@@ -315,9 +330,9 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
       a += sm_acc[w][h][d] * wt;
     }
     if (FINAL) {
-      out[((int64_t)b * num_heads + g * G + h) * kPaD + d] = (f16)(lsum > 0.f ? a / lsum : 0.f);
+      out[((int64_t)b * num_heads + g * group + h) * kPaD + d] = (f16)(lsum > 0.f ? a / lsum : 0.f);
     } else {
-      const int64_t slot = ((int64_t)b * num_heads + g * G + h) * max_splits + split;
+      const int64_t slot = ((int64_t)b * num_heads + g * group + h) * max_splits + split;
       part_o[slot * kPaD + d] = a;
       if (d == 0) {
         part_ml[slot * 2 + 0] = mx;
@@ -327,7 +342,8 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
   }
 }
 
-// grid = (Hq, bs), block = 128: one thread per output element.
+// grid = (Hq, bs), block = head_dim: one thread per output element.
+template <int kPaD>
 __global__ __launch_bounds__(kPaD) void pa_decode_merge(const float* __restrict__ part_o,
                                                         const float* __restrict__ part_ml,
                                                         const int32_t* __restrict__ context_lens,
@@ -356,7 +372,7 @@ __global__ __launch_bounds__(kPaD) void pa_decode_merge(const float* __restrict_
   o[out] = (f16)(lsum > 0.f ? a / lsum : 0.f);
 }
 
-template <int G>
+template <int kPaD, int GMAX>
 static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t* bt,
                       const int32_t* cl, f16* o, float* part_o, float* part_ml, int bs,
                       int num_heads, int num_kv_heads, int block_size, int max_blocks_per_seq,
@@ -364,16 +380,16 @@ static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t*
   const float scale_log2 = kLog2e / __builtin_sqrtf((float)kPaD);
   dim3 grid((unsigned)ch.max_splits, (unsigned)num_kv_heads, (unsigned)bs);
   if (ch.max_splits == 1) {
-    pa_decode_partial<G, true><<<grid, kPaWaves * kWave, 0, s>>>(
+    pa_decode_partial<kPaD, GMAX, true><<<grid, kPaWaves * kWave, 0, s>>>(
         q, kc, vc, bt, cl, part_o, part_ml, o, num_kv_heads, block_size, max_blocks_per_seq,
-        ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks);
+        ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads);
     return;
   }
-  pa_decode_partial<G, false><<<grid, kPaWaves * kWave, 0, s>>>(
+  pa_decode_partial<kPaD, GMAX, false><<<grid, kPaWaves * kWave, 0, s>>>(
       q, kc, vc, bt, cl, part_o, part_ml, o, num_kv_heads, block_size, max_blocks_per_seq,
-      ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks);
+      ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads);
   dim3 mgrid((unsigned)num_heads, (unsigned)bs);
-  pa_decode_merge<<<mgrid, kPaD, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
+  pa_decode_merge<kPaD><<<mgrid, kPaD, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
                                          ch.max_splits);
 }
 
@@ -467,9 +483,9 @@ static bool pa_args_valid(int64_t bs, int64_t num_heads, int64_t num_kv_heads, i
 // Shapes served by the MFMA kernel; everything else that is valid takes the generic kernel.
 static bool pa_fast_shape(int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
                           int64_t block_size) {
-  if (head_dim != kPaD || block_size % kPaStep != 0) return false;
-  const int64_t group = num_heads / num_kv_heads;
-  return group == 1 || group == 2 || group == 4 || group == 8 || group == 16;
+  if ((head_dim != 64 && head_dim != 128 && head_dim != 256) || block_size % 16 != 0) return false;
+  // the cross-wave merge keeps 8 x group x head_dim floats in LDS: at most 66 KB
+  return (num_heads / num_kv_heads) * head_dim <= 16 * 128;
 }
 
 }  // namespace aops
@@ -482,7 +498,7 @@ extern "C" size_t aops_paged_attention_workspace(int64_t bs, int64_t num_heads,
     return 0;
   if (!pa_fast_shape(num_heads, num_kv_heads, head_dim, block_size)) return 16;  // not used
   const PaChunking ch = pa_chunking(bs, num_kv_heads, block_size, max_blocks_per_seq);
-  return (size_t)bs * (size_t)num_heads * (size_t)ch.max_splits * (kPaD + 2) * sizeof(float);
+  return (size_t)bs * (size_t)num_heads * (size_t)ch.max_splits * (size_t)(head_dim + 2) * sizeof(float);
 }
 
 extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
@@ -519,22 +535,31 @@ extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
   if (!workspace || workspace_bytes < need) return AOPS_ERR_WORKSPACE;
   const PaChunking ch = pa_chunking(bs, num_kv_heads, block_size, max_blocks_per_seq);
   float* part_o = static_cast<float*>(workspace);
-  float* part_ml = part_o + (size_t)bs * num_heads * ch.max_splits * kPaD;
-#define AOPS_PA_CASE(G)                                                                        \
-  case G:                                                                                      \
-    pa_launch<G>(qp, kc, vc, block_tables, context_lens, op, part_o, part_ml, (int)bs,         \
-                 (int)num_heads, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq,  \
-                 ch, s, (int)num_blocks);                                                      \
+  float* part_ml = part_o + (size_t)bs * num_heads * ch.max_splits * head_dim;
+#define AOPS_PA_CASE(D, G)                                                                      \
+  case G:                                                                                       \
+    pa_launch<D, G>(qp, kc, vc, block_tables, context_lens, op, part_o, part_ml, (int)bs,       \
+                    (int)num_heads, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq, \
+                    ch, s, (int)num_blocks);                                                    \
     break;
-  switch (num_heads / num_kv_heads) {
-    AOPS_PA_CASE(1)
-    AOPS_PA_CASE(2)
-    AOPS_PA_CASE(4)
-    AOPS_PA_CASE(8)
-    AOPS_PA_CASE(16)
-    default:
-      return AOPS_ERR_INVALID_ARGUMENT;
+#define AOPS_PA_GROUPS(D)     \
+  switch (gmax) {             \
+    AOPS_PA_CASE(D, 1)        \
+    AOPS_PA_CASE(D, 2)        \
+    AOPS_PA_CASE(D, 4)        \
+    AOPS_PA_CASE(D, 8)        \
+    AOPS_PA_CASE(D, 16)       \
   }
+  const int64_t group = num_heads / num_kv_heads;
+  const int gmax = group <= 1 ? 1 : group <= 2 ? 2 : group <= 4 ? 4 : group <= 8 ? 8 : 16;
+  if (head_dim == 64) {
+    AOPS_PA_GROUPS(64)
+  } else if (head_dim == 128) {
+    AOPS_PA_GROUPS(128)
+  } else {
+    AOPS_PA_GROUPS(256)
+  }
+#undef AOPS_PA_GROUPS
 #undef AOPS_PA_CASE
   return record_launch_status(hipGetLastError());
 }

@@ -542,6 +542,57 @@ def test_paged_attention_other_shapes(ops, dev, B, Hq, Hkv, D, P, lens):
     assert (o.float() - ref.float()).abs().max() < 3e-3
 
 
+@pytest.mark.parametrize(
+    "B,Hq,Hkv,P,lens",
+    [
+        (3, 24, 8, 128, [130, 700, 2500]),      # 3 query heads per kv head
+        (2, 10, 2, 64, [64, 1000]),             # 5
+        (2, 12, 2, 128, [1, 300]),              # 6
+        (2, 14, 2, 32, [31, 33]),               # 7
+        (2, 24, 2, 128, [257, 4000]),           # 12
+        (4, 32, 8, 16, [16, 17, 300, 1]),       # 16-token pages: the two halves of a step lie in different pages
+        (3, 32, 8, 48, [48, 96, 1000]),         # page size an odd multiple of 16; lengths that fill the last page
+        (2, 6, 2, 80, [79, 2000]),              # 3 heads per kv head on 80-token pages
+        (2, 16, 4, 144, [144, 145]),
+    ],
+)
+def test_paged_attention_matrix_core_path_any_group_and_page_size(ops, dev, B, Hq, Hkv, P, lens):
+    """head_dim 128 takes the matrix-core kernel for every group size up to 16 and every page size that is a multiple
+    of 16; unused cache slots hold NaN and unused table entries -1."""
+    import ascend910a_extras.ascend910a_extras_C as C
+
+    assert C._lib.aops_paged_attention_workspace(B, Hq, Hkv, 128, P, 64) > 16   # not the generic kernel
+    case = _paged_case(B, Hq, Hkv, 128, P, lens, seed=9, poison=True)
+    o = _run_pa(ops, dev, case)
+    ref = R.paged_attention_ref(*case)
+    assert not torch.isnan(o).any()
+    torch.testing.assert_close(o.float(), ref.float(), **TOL)
+    assert (o.float() - ref.float()).abs().max() < 3e-3
+
+
+@pytest.mark.parametrize(
+    "B,Hq,Hkv,D,P,lens",
+    [
+        (4, 32, 8, 64, 128, [512, 4096, 1000, 37]),     # head_dim 64, sequences split into chunks
+        (3, 16, 2, 64, 16, [1, 50, 2000]),              # 8 heads per kv head on 16-token pages
+        (2, 12, 4, 64, 48, [48, 300]),
+        (3, 16, 8, 256, 128, [130, 3000, 1]),           # head_dim 256
+        (2, 16, 2, 256, 32, [33, 700]),                 # 8 heads per kv head: the largest group at 256
+        (2, 3, 1, 256, 64, [64, 65]),
+    ],
+)
+def test_paged_attention_matrix_core_path_other_head_sizes(ops, dev, B, Hq, Hkv, D, P, lens):
+    import ascend910a_extras.ascend910a_extras_C as C
+
+    assert C._lib.aops_paged_attention_workspace(B, Hq, Hkv, D, P, 64) > 16   # not the generic kernel
+    case = _paged_case(B, Hq, Hkv, D, P, lens, seed=13, poison=True)
+    o = _run_pa(ops, dev, case)
+    ref = R.paged_attention_ref(*case)
+    assert o.shape == (B, Hq, D) and not torch.isnan(o).any()
+    torch.testing.assert_close(o.float(), ref.float(), **TOL)
+    assert (o.float() - ref.float()).abs().max() < 3e-3
+
+
 def test_paged_attention_ignores_garbage_and_unused_table_entries(ops, dev):
     lens = [5, 130, 257, 1]
     clean = _paged_case(4, 32, 8, 128, 128, lens, seed=1, max_pages=6)
