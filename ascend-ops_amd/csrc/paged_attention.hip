@@ -43,8 +43,11 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 struct PaChunking {
   int chunk_tokens;  // tokens per workgroup (multiple of kPaWaves*kPaStep)
-  int max_splits;    // chunks needed for the longest possible context
+  int max_splits;    // partial-result slots per (sequence, head): chunks of the longest possible context
+  int balanced_wgs;  // > 0: workgroups per kv head of the balanced partition (see pa_decode_balanced)
 };
+
+constexpr int kPaUnit = kPaWaves * kPaStep;  // 256 tokens: one step of every wave
 
 static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_size,
                               int64_t max_blocks_per_seq) {
@@ -69,6 +72,22 @@ static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_si
   c.chunk_tokens = chunk;
   c.max_splits = (int)((max_len + chunk - 1) / chunk);
   if (c.max_splits < 1) c.max_splits = 1;
+  c.balanced_wgs = 0;
+  // Small batches: fixed chunks of a few long sequences either leave CUs idle or, cut finer, pay
+  // the per-workgroup start-up many times over.  With fewer than two (sequence, kv head) pairs per
+  // CU the token stream is cut into one equal share per CU instead.
+  static const int balanced_env = [] {
+    const char* e = getenv("AOPS_PA_BALANCED");  // tuning aid: 0 = off, n = n workgroups in total
+    return e ? atoi(e) : -1;
+  }();
+  constexpr int64_t kCus = 256;
+  if (!forced && balanced_env != 0 && bs <= kWave && bs * num_kv_heads < 2 * kCus && max_units >= 2) {
+    const int64_t total = balanced_env > 0 ? balanced_env : kCus;
+    int64_t wgs = (total + num_kv_heads - 1) / num_kv_heads;
+    if (wgs > bs * max_units) wgs = bs * max_units;  // never more shares than units
+    c.balanced_wgs = (int)wgs;
+    c.max_splits = (int)(wgs < max_units ? wgs : max_units);
+  }
   return c;
 }
 
@@ -170,47 +189,21 @@ __device__ __forceinline__ void pa_accumulate(const PaRegs<NS>& v, const f16x8 (
   }
 }
 
-// grid = (max_splits, Hkv, bs), block = 8 waves.  `group` = query heads per kv head, GMAX = the
-// power of two it is rounded up to (<= 16; sizes the LDS arrays).
-// FINAL: the chunk is the whole sequence, so the normalised output is written directly.
+// One chunk of one (sequence b, kv head g): tokens chunk_start .. chunk_start + chunk_len - 1, the
+// steps dealt round robin to the eight waves, which are merged through LDS at the end.  `group` =
+// query heads per kv head, GMAX = the power of two it is rounded up to (<= 16; sizes the LDS
+// arrays).  FINAL: the chunk is the whole sequence, so the normalised output is written directly;
+// otherwise the partial result goes to slot `split` of the (sequence, head)'s max_splits slots.
+// Called by all threads of the workgroup with uniform arguments.
 template <int D, int GMAX, bool FINAL>
-__global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
+__device__ __forceinline__ void pa_process_chunk(
     const f16* __restrict__ q, const f16* __restrict__ key_cache,
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
-    const int32_t* __restrict__ context_lens, float* __restrict__ part_o,
-    float* __restrict__ part_ml, f16* __restrict__ out, int num_kv_heads, int block_size, int max_blocks_per_seq,
-    int chunk_tokens, int max_splits, float scale_log2, int num_blocks, int group) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, f16* __restrict__ out, int b, int g,
+    int context_len, int chunk_start, int chunk_len, int split, int num_kv_heads, int block_size,
+    int max_blocks_per_seq, int max_splits, float scale_log2, int num_blocks, int group) {
   constexpr int kPaD = D;
   constexpr int NS = D / 32;
-  const int split = blockIdx.x;
-  const int g = blockIdx.y;
-  // Workgroups are handed out in index order, so they take the sequences longest first: with
-  // one resident workgroup per CU the short sequences then fill the gaps the long ones leave
-  // (longest-processing-time-first).  For batches of up to 64 sequences every wave finds the
-  // sequence of rank blockIdx.z by comparing the lengths held one per lane.
-  int b = blockIdx.z;
-  if (gridDim.z <= kWave) {
-    const int ln = threadIdx.x & (kWave - 1);
-    const int mine = ln < (int)gridDim.z ? context_lens[ln] : -0x7fffffff - 1;
-    int rank = 0;
-    for (int j = 0; j < (int)gridDim.z; ++j) {
-      const int other = __builtin_amdgcn_readlane(mine, j);
-      rank += (other > mine || (other == mine && j < ln)) ? 1 : 0;
-    }
-    const uint64_t hit = __ballot(rank == (int)blockIdx.z && ln < (int)gridDim.z);
-    if (hit) b = __builtin_ctzll(hit);  // exactly one lane has each rank
-  }
-  // a length beyond the block table would walk off the table row
-  const int context_len = min(context_lens[b], max_blocks_per_seq * block_size);
-  const int chunk_start = split * chunk_tokens;
-  if (chunk_start >= context_len) {
-    if (FINAL) {  // empty sequence: zeros
-      for (int e = threadIdx.x; e < group * kPaD; e += kPaWaves * kWave)
-        out[((int64_t)b * num_kv_heads * group + g * group) * kPaD + e] = (f16)0.f;
-    }
-    return;
-  }
-  const int chunk_len = min(context_len - chunk_start, chunk_tokens);
   const int nsteps = (chunk_len + kPaStep - 1) / kPaStep;
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -342,13 +335,126 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
   }
 }
 
+// grid = (max_splits, Hkv, bs), block = 8 waves: one chunk of chunk_tokens tokens per workgroup.
+template <int D, int GMAX, bool FINAL>
+__global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
+    const f16* __restrict__ q, const f16* __restrict__ key_cache,
+    const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
+    const int32_t* __restrict__ context_lens, float* __restrict__ part_o,
+    float* __restrict__ part_ml, f16* __restrict__ out, int num_kv_heads, int block_size, int max_blocks_per_seq,
+    int chunk_tokens, int max_splits, float scale_log2, int num_blocks, int group) {
+  const int split = blockIdx.x;
+  const int g = blockIdx.y;
+  // Workgroups are handed out in index order, so they take the sequences longest first: with
+  // one resident workgroup per CU the short sequences then fill the gaps the long ones leave
+  // (longest-processing-time-first).  For batches of up to 64 sequences every wave finds the
+  // sequence of rank blockIdx.z by comparing the lengths held one per lane.
+  int b = blockIdx.z;
+  if (gridDim.z <= kWave) {
+    const int ln = threadIdx.x & (kWave - 1);
+    const int mine = ln < (int)gridDim.z ? context_lens[ln] : -0x7fffffff - 1;
+    int rank = 0;
+    for (int j = 0; j < (int)gridDim.z; ++j) {
+      const int other = __builtin_amdgcn_readlane(mine, j);
+      rank += (other > mine || (other == mine && j < ln)) ? 1 : 0;
+    }
+    const uint64_t hit = __ballot(rank == (int)blockIdx.z && ln < (int)gridDim.z);
+    if (hit) b = __builtin_ctzll(hit);  // exactly one lane has each rank
+  }
+  // a length beyond the block table would walk off the table row
+  const int context_len = min(context_lens[b], max_blocks_per_seq * block_size);
+  const int chunk_start = split * chunk_tokens;
+  if (chunk_start >= context_len) {
+    if (FINAL) {  // empty sequence: zeros
+      for (int e = threadIdx.x; e < group * D; e += kPaWaves * kWave)
+        out[((int64_t)b * num_kv_heads * group + g * group) * D + e] = (f16)0.f;
+    }
+    return;
+  }
+  pa_process_chunk<D, GMAX, FINAL>(q, key_cache, value_cache, block_tables, part_o, part_ml, out, b, g,
+                                   context_len, chunk_start, min(context_len - chunk_start, chunk_tokens),
+                                   split, num_kv_heads, block_size, max_blocks_per_seq, max_splits,
+                                   scale_log2, num_blocks, group);
+}
+
+// Balanced partition for batches of up to 64 sequences.  Lane l of every wave holds sequence l:
+// its length, its number of 256-token units, and the number of units in front of it.
+struct PaUnits {
+  int len;     // context length, clamped to [0, table capacity]
+  int units;   // ceil(len / 256)
+  int before;  // units of the sequences 0 .. l-1
+  int total;   // units of the whole batch
+};
+
+__device__ __forceinline__ PaUnits pa_units(const int32_t* __restrict__ context_lens, int bs, int max_len) {
+  const int lane = threadIdx.x & (kWave - 1);
+  PaUnits r;
+  r.len = lane < bs ? min(max(context_lens[lane], 0), max_len) : 0;
+  r.units = (r.len + kPaUnit - 1) / kPaUnit;
+  int incl = r.units;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int up = __shfl_up(incl, d);
+    if (lane >= d) incl += up;
+  }
+  r.before = incl - r.units;
+  r.total = __shfl(incl, kWave - 1);
+  return r;
+}
+
+// Share w of `wgs` covers units [w*total/wgs, (w+1)*total/wgs); this is the share that holds unit x.
+__device__ __forceinline__ int pa_share_of(int x, int wgs, int total) {
+  return (int)((((int64_t)x + 1) * wgs - 1) / total);
+}
+
+// grid = (wgs, Hkv), block = 8 waves.  Workgroup w walks through its share of the batch's units,
+// sequence by sequence; the part of sequence b it covers becomes partial result number
+// w - (share holding b's first unit) of that sequence.
+template <int D, int GMAX>
+__global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_balanced(
+    const f16* __restrict__ q, const f16* __restrict__ key_cache,
+    const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
+    const int32_t* __restrict__ context_lens, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int bs, int num_kv_heads, int block_size, int max_blocks_per_seq,
+    int max_splits, float scale_log2, int num_blocks, int group) {
+  const int w = blockIdx.x;
+  const int g = blockIdx.y;
+  const PaUnits pu = pa_units(context_lens, bs, max_blocks_per_seq * block_size);
+  // no more shares than units: every share then holds at least one unit, and the shares of a
+  // sequence are consecutive
+  const int wgs = min((int)gridDim.x, pu.total);
+  if (w >= wgs) return;
+  const int lo = (int)((int64_t)w * pu.total / wgs);
+  const int hi = (int)((int64_t)(w + 1) * pu.total / wgs);
+  int cur = lo;
+  while (cur < hi) {
+    // the sequence that holds unit cur (exactly one lane)
+    const uint64_t hit = __ballot(pu.units > 0 && pu.before <= cur && cur < pu.before + pu.units);
+    if (hit == 0) break;  // cannot happen: the units of the sequences tile [0, total)
+    const int b = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(hit));
+    const int before = __builtin_amdgcn_readlane(pu.before, b);
+    const int units = __builtin_amdgcn_readlane(pu.units, b);
+    const int len = __builtin_amdgcn_readlane(pu.len, b);
+    const int seg_end = min(hi, before + units);
+    const int tok0 = (cur - before) * kPaUnit;
+    const int tok1 = min((seg_end - before) * kPaUnit, len);
+    const int slot = w - pa_share_of(before, wgs, pu.total);
+    pa_process_chunk<D, GMAX, false>(q, key_cache, value_cache, block_tables, part_o, part_ml, nullptr, b, g,
+                                     len, tok0, tok1 - tok0, slot, num_kv_heads, block_size,
+                                     max_blocks_per_seq, max_splits, scale_log2, num_blocks, group);
+    cur = seg_end;
+    if (cur < hi) __syncthreads();  // the LDS arrays of the chunk are reused
+  }
+}
+
 // grid = (Hq, bs), block = head_dim: one thread per output element.
 template <int kPaD>
 __global__ __launch_bounds__(kPaD) void pa_decode_merge(const float* __restrict__ part_o,
                                                         const float* __restrict__ part_ml,
                                                         const int32_t* __restrict__ context_lens,
                                                         f16* __restrict__ o, int num_heads,
-                                                        int chunk_tokens, int max_splits) {
+                                                        int chunk_tokens, int max_splits, int balanced_wgs,
+                                                        int bs, int max_len) {
   const int h = blockIdx.x;
   const int b = blockIdx.y;
   const int d = threadIdx.x;
@@ -358,7 +464,16 @@ __global__ __launch_bounds__(kPaD) void pa_decode_merge(const float* __restrict_
     o[out] = (f16)0.f;
     return;
   }
-  int nsplit = (context_len + chunk_tokens - 1) / chunk_tokens;
+  int nsplit;
+  if (balanced_wgs > 0) {  // partial results of the shares that hold the sequence's first and last unit
+    const PaUnits pu = pa_units(context_lens, bs, max_len);
+    const int before = __builtin_amdgcn_readlane(pu.before, b);
+    const int units = __builtin_amdgcn_readlane(pu.units, b);
+    const int wgs = min(balanced_wgs, pu.total);
+    nsplit = pa_share_of(before + units - 1, wgs, pu.total) - pa_share_of(before, wgs, pu.total) + 1;
+  } else {
+    nsplit = (context_len + chunk_tokens - 1) / chunk_tokens;
+  }
   if (nsplit > max_splits) nsplit = max_splits;
   const int64_t base = ((int64_t)b * num_heads + h) * max_splits;
   float mx = kNegBig;
@@ -378,6 +493,17 @@ static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t*
                       int num_heads, int num_kv_heads, int block_size, int max_blocks_per_seq,
                       PaChunking ch, hipStream_t s, int num_blocks) {
   const float scale_log2 = kLog2e / __builtin_sqrtf((float)kPaD);
+  if (ch.balanced_wgs > 0) {
+    dim3 bgrid((unsigned)ch.balanced_wgs, (unsigned)num_kv_heads);
+    pa_decode_balanced<kPaD, GMAX><<<bgrid, kPaWaves * kWave, 0, s>>>(
+        q, kc, vc, bt, cl, part_o, part_ml, bs, num_kv_heads, block_size, max_blocks_per_seq,
+        ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads);
+    dim3 mgrid((unsigned)num_heads, (unsigned)bs);
+    pa_decode_merge<kPaD><<<mgrid, kPaD, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
+                                           ch.max_splits, ch.balanced_wgs, bs,
+                                           max_blocks_per_seq * block_size);
+    return;
+  }
   dim3 grid((unsigned)ch.max_splits, (unsigned)num_kv_heads, (unsigned)bs);
   if (ch.max_splits == 1) {
     pa_decode_partial<kPaD, GMAX, true><<<grid, kPaWaves * kWave, 0, s>>>(
@@ -390,7 +516,7 @@ static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t*
       ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads);
   dim3 mgrid((unsigned)num_heads, (unsigned)bs);
   pa_decode_merge<kPaD><<<mgrid, kPaD, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
-                                         ch.max_splits);
+                                         ch.max_splits, 0, bs, max_blocks_per_seq * block_size);
 }
 
 // Generic path for every other shape (head_dim a multiple of 16 up to 256, any block size, any

@@ -593,6 +593,34 @@ def test_paged_attention_matrix_core_path_other_head_sizes(ops, dev, B, Hq, Hkv,
     assert (o.float() - ref.float()).abs().max() < 3e-3
 
 
+@pytest.mark.parametrize(
+    "B,Hq,Hkv,P,maxlen,seed",
+    [
+        (40, 32, 8, 128, 3000, 1),     # 320 (sequence, kv head) pairs: more units than shares, several sequences per share
+        (63, 8, 2, 64, 1200, 2),       # 128 shares per kv head
+        (5, 4, 1, 128, 9000, 3),       # 256 shares for five sequences: long sequences cut into many partial results
+        (33, 16, 4, 16, 700, 4),       # 16-token pages
+        (12, 32, 8, 128, 255, 5),      # every sequence shorter than one 256-token unit
+    ],
+)
+def test_paged_attention_balanced_partition(ops, dev, B, Hq, Hkv, P, maxlen, seed):
+    """Batches with fewer than two (sequence, kv head) pairs per CU: the token stream is cut into equal shares of
+    256-token units, one per workgroup, whatever the sequence boundaries; a share may hold the end of one sequence,
+    whole sequences and the start of another.  Empty sequences in between, NaN in unused slots."""
+    import random
+    rnd = random.Random(seed)
+    lens = [rnd.choice([0, 1, 255, 256, 257, rnd.randint(1, maxlen), rnd.randint(1, maxlen)]) for _ in range(B)]
+    lens[rnd.randrange(B)] = maxlen
+    case = _paged_case(B, Hq, Hkv, 128, P, lens, seed=seed, poison=True)
+    o = _run_pa(ops, dev, case)
+    ref = R.paged_attention_ref(*case)
+    assert not torch.isnan(o).any()
+    torch.testing.assert_close(o.float(), ref.float(), **TOL)
+    assert (o.float() - ref.float()).abs().max() < 3e-3
+    # deterministic: the partial results are merged in a fixed order
+    assert torch.equal(_run_pa(ops, dev, case), o)
+
+
 def test_paged_attention_ignores_garbage_and_unused_table_entries(ops, dev):
     lens = [5, 130, 257, 1]
     clean = _paged_case(4, 32, 8, 128, 128, lens, seed=1, max_pages=6)
