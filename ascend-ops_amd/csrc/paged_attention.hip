@@ -335,6 +335,25 @@ __device__ __forceinline__ void pa_process_chunk(
   }
 }
 
+constexpr int kPaRankMax = 1024;
+
+// One workgroup: order[r] = the sequence with the r-th longest context (ties by index).
+__global__ __launch_bounds__(kPaRankMax) void pa_rank_sequences(const int32_t* __restrict__ context_lens,
+                                                                int bs, int32_t* __restrict__ order) {
+  __shared__ int lens[kPaRankMax];
+  const int t = threadIdx.x;
+  const int mine = t < bs ? context_lens[t] : 0;
+  lens[t] = mine;
+  __syncthreads();
+  if (t >= bs) return;
+  int rank = 0;
+  for (int j = 0; j < bs; ++j) {
+    const int other = lens[j];
+    rank += (other > mine || (other == mine && j < t)) ? 1 : 0;
+  }
+  order[rank] = t;
+}
+
 // grid = (max_splits, Hkv, bs), block = 8 waves: one chunk of chunk_tokens tokens per workgroup.
 template <int D, int GMAX, bool FINAL>
 __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
@@ -342,14 +361,16 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ context_lens, float* __restrict__ part_o,
     float* __restrict__ part_ml, f16* __restrict__ out, int num_kv_heads, int block_size, int max_blocks_per_seq,
-    int chunk_tokens, int max_splits, float scale_log2, int num_blocks, int group) {
+    int chunk_tokens, int max_splits, float scale_log2, int num_blocks, int group,
+    const int32_t* __restrict__ order) {
   const int split = blockIdx.x;
   const int g = blockIdx.y;
   // Workgroups are handed out in index order, so they take the sequences longest first: with
   // one resident workgroup per CU the short sequences then fill the gaps the long ones leave
   // (longest-processing-time-first).  For batches of up to 64 sequences every wave finds the
-  // sequence of rank blockIdx.z by comparing the lengths held one per lane.
-  int b = blockIdx.z;
+  // sequence of rank blockIdx.z by comparing the lengths held one per lane; larger batches (up to
+  // kPaRankMax sequences) get the order from pa_rank_sequences.
+  int b = order ? order[blockIdx.z] : (int)blockIdx.z;
   if (gridDim.z <= kWave) {
     const int ln = threadIdx.x & (kWave - 1);
     const int mine = ln < (int)gridDim.z ? context_lens[ln] : -0x7fffffff - 1;
@@ -491,7 +512,7 @@ template <int kPaD, int GMAX>
 static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t* bt,
                       const int32_t* cl, f16* o, float* part_o, float* part_ml, int bs,
                       int num_heads, int num_kv_heads, int block_size, int max_blocks_per_seq,
-                      PaChunking ch, hipStream_t s, int num_blocks) {
+                      PaChunking ch, hipStream_t s, int num_blocks, int32_t* order) {
   const float scale_log2 = kLog2e / __builtin_sqrtf((float)kPaD);
   if (ch.balanced_wgs > 0) {
     dim3 bgrid((unsigned)ch.balanced_wgs, (unsigned)num_kv_heads);
@@ -505,15 +526,17 @@ static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t*
     return;
   }
   dim3 grid((unsigned)ch.max_splits, (unsigned)num_kv_heads, (unsigned)bs);
+  if (bs <= kWave || bs > kPaRankMax) order = nullptr;  // ranked inside the kernel / not ranked at all
+  if (order) pa_rank_sequences<<<1, kPaRankMax, 0, s>>>(cl, bs, order);
   if (ch.max_splits == 1) {
     pa_decode_partial<kPaD, GMAX, true><<<grid, kPaWaves * kWave, 0, s>>>(
         q, kc, vc, bt, cl, part_o, part_ml, o, num_kv_heads, block_size, max_blocks_per_seq,
-        ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads);
+        ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads, order);
     return;
   }
   pa_decode_partial<kPaD, GMAX, false><<<grid, kPaWaves * kWave, 0, s>>>(
       q, kc, vc, bt, cl, part_o, part_ml, o, num_kv_heads, block_size, max_blocks_per_seq,
-      ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads);
+      ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads, order);
   dim3 mgrid((unsigned)num_heads, (unsigned)bs);
   pa_decode_merge<kPaD><<<mgrid, kPaD, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
                                          ch.max_splits, 0, bs, max_blocks_per_seq * block_size);
@@ -624,7 +647,9 @@ extern "C" size_t aops_paged_attention_workspace(int64_t bs, int64_t num_heads,
     return 0;
   if (!pa_fast_shape(num_heads, num_kv_heads, head_dim, block_size)) return 16;  // not used
   const PaChunking ch = pa_chunking(bs, num_kv_heads, block_size, max_blocks_per_seq);
-  return (size_t)bs * (size_t)num_heads * (size_t)ch.max_splits * (size_t)(head_dim + 2) * sizeof(float);
+  // partial results, then one int per sequence (the length order of batches above 64 sequences)
+  return (size_t)bs * (size_t)num_heads * (size_t)ch.max_splits * (size_t)(head_dim + 2) * sizeof(float) +
+         (size_t)bs * sizeof(int32_t);
 }
 
 extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
@@ -662,11 +687,12 @@ extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
   const PaChunking ch = pa_chunking(bs, num_kv_heads, block_size, max_blocks_per_seq);
   float* part_o = static_cast<float*>(workspace);
   float* part_ml = part_o + (size_t)bs * num_heads * ch.max_splits * head_dim;
+  int32_t* order = reinterpret_cast<int32_t*>(part_ml + (size_t)bs * num_heads * ch.max_splits * 2);
 #define AOPS_PA_CASE(D, G)                                                                      \
   case G:                                                                                       \
     pa_launch<D, G>(qp, kc, vc, block_tables, context_lens, op, part_o, part_ml, (int)bs,       \
                     (int)num_heads, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq, \
-                    ch, s, (int)num_blocks);                                                    \
+                    ch, s, (int)num_blocks, order);                                             \
     break;
 #define AOPS_PA_GROUPS(D)     \
   switch (gmax) {             \

@@ -56,11 +56,12 @@ def test_workspace_query_without_gpu():
 
     # config 5 shape: 64 x 32 heads, 8 kv heads, D=128, P=128, 32 pages; one (max, sum, 128 floats)
     # record per (sequence, head, chunk), the number of chunks being the library's choice
-    n = C._lib.aops_paged_attention_workspace(64, 32, 8, 128, 128, 32)
+    # plus one int per sequence
+    n = C._lib.aops_paged_attention_workspace(64, 32, 8, 128, 128, 32) - 64 * 4
     per_chunk = 64 * 32 * 130 * 4
     assert n >= per_chunk and n % per_chunk == 0 and n // per_chunk <= 32
     # a single short sequence is split into more chunks than a large batch
-    n1 = C._lib.aops_paged_attention_workspace(1, 32, 8, 128, 128, 32)
+    n1 = C._lib.aops_paged_attention_workspace(1, 32, 8, 128, 128, 32) - 4
     assert n1 // (32 * 130 * 4) > n // per_chunk
     assert C._lib.aops_paged_attention_workspace(64, 32, 8, 100, 128, 32) == 0  # head_dim % 16 != 0
     assert C._lib.aops_paged_attention_workspace(64, 32, 8, 512, 128, 32) == 0  # head_dim > 256

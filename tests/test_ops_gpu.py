@@ -507,18 +507,21 @@ def test_paged_attention_clamps_block_table_entries(ops, dev, D, P, Hq, Hkv):
     torch.testing.assert_close(o[[0, 2]].float(), good[[0, 2]].float(), **TOL)
 
 
-def test_paged_attention_batch_larger_than_a_wave(ops, dev):
-    """More than 64 sequences: the longest-first ordering of the workgroups (one length per lane) is off and the
-    sequences are taken in index order; several chunks per sequence when the batch alone fills the chip."""
+@pytest.mark.parametrize("B,Hq,Hkv,P", [(150, 8, 2, 64), (70, 4, 1, 128), (1030, 2, 1, 32)])
+def test_paged_attention_batch_larger_than_a_wave(ops, dev, B, Hq, Hkv, P):
+    """More than 64 sequences: a one-workgroup kernel ranks the sequences by length (up to 1024 of them; beyond that
+    they are taken in index order) and the workgroups take them longest first; with few kv heads the sequences are
+    also cut into several chunks.  Ties, empty sequences and one very long sequence included."""
     rnd = torch.Generator().manual_seed(12)
-    B = 150
     lens = torch.randint(0, 600, (B,), generator=rnd).tolist()
     lens[3] = 0
-    lens[77] = 2500
-    case = _paged_case(B, 8, 2, 128, 64, lens, seed=12)
+    lens[5] = lens[6] = lens[60] = 333
+    lens[B // 2] = 2500
+    case = _paged_case(B, Hq, Hkv, 128, P, lens, seed=12)
     o = _run_pa(ops, dev, case)
     ref = R.paged_attention_ref(*case)
     torch.testing.assert_close(o.float(), ref.float(), **TOL)
+    assert (o.float() - ref.float()).abs().max() < 3e-3
 
 
 @pytest.mark.parametrize(
