@@ -70,15 +70,19 @@ def time_graph(calls, min_launches=200, trials=5):
     for c in calls:
         c()
     torch.cuda.synchronize()
+    # at least 32 launches per graph: the gap between two replays is then shared by many launches
+    rounds = max(1, -(-32 // len(calls)))
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        for c in calls:
-            c()
-    reps = max(1, -(-min_launches // len(calls)))
+        for _ in range(rounds):
+            for c in calls:
+                c()
+    launches = rounds * len(calls)
+    reps = max(1, -(-min_launches // launches))
     graph.replay()
     per = []
     for _ in range(trials):
-        per.append(_events_ms(graph.replay, reps) * 1e3 / (reps * len(calls)))
+        per.append(_events_ms(graph.replay, reps) * 1e3 / (reps * launches))
     del graph
     return statistics.median(per), min(per)
 
