@@ -275,6 +275,47 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
   st128_stream(out + (t * vec_per_row + c) * 8, o);
 }
 
+// Routing tables of a few tokens (at most kSmallSort ids): one workgroup, one launch.  Thread t
+// ranks id t by counting the ids that sort in front of it (smaller bucket, or the same bucket and
+// a smaller index: stable), thread e counts the ids of experts 0..e for group_list; both walk the
+// buckets held in LDS.
+constexpr int kSmallSort = 128;  // quadratic work on one CU: beyond this the sliced sort is faster
+
+__global__ __launch_bounds__(kSmallSort) void moe_sort_small_kernel(
+    const int32_t* __restrict__ ids, int n, int num_experts, int32_t* __restrict__ sorted_idx,
+    int32_t* __restrict__ inverse_idx, int64_t* __restrict__ group_list) {
+  __shared__ __attribute__((aligned(16))) int32_t bucket[kSmallSort];
+  const int t = threadIdx.x;
+  // entries past n hold a bucket larger than any real one: they are never counted
+  const int mine = t < n ? moe_bucket(ids[t], num_experts) : num_experts + 1;
+  bucket[t] = mine;
+  __syncthreads();
+  const int n4 = (n + 3) / 4;
+  const int4* b4 = reinterpret_cast<const int4*>(bucket);
+  if (t < n) {
+    int rank = 0;
+#pragma unroll 8
+    for (int j = 0; j < n4; ++j) {  // same address in every lane: one LDS broadcast per four ids
+      const int4 o = b4[j];
+      rank += (o.x < mine || (o.x == mine && 4 * j < t)) ? 1 : 0;
+      rank += (o.y < mine || (o.y == mine && 4 * j + 1 < t)) ? 1 : 0;
+      rank += (o.z < mine || (o.z == mine && 4 * j + 2 < t)) ? 1 : 0;
+      rank += (o.w < mine || (o.w == mine && 4 * j + 3 < t)) ? 1 : 0;
+    }
+    sorted_idx[rank] = t;
+    if (inverse_idx) inverse_idx[t] = rank;
+  }
+  for (int e = t; e < num_experts; e += kSmallSort) {
+    int upto = 0;
+#pragma unroll 8
+    for (int j = 0; j < n4; ++j) {
+      const int4 o = b4[j];
+      upto += (o.x <= e ? 1 : 0) + (o.y <= e ? 1 : 0) + (o.z <= e ? 1 : 0) + (o.w <= e ? 1 : 0);
+    }
+    group_list[e] = upto;
+  }
+}
+
 static int64_t moe_slices(int64_t n) { return (n + kSlice - 1) / kSlice; }
 
 }  // namespace aops
@@ -296,6 +337,11 @@ extern "C" int aops_moe_sort_i32(const int32_t* expert_ids, int64_t n, int64_t n
   const size_t need = aops_moe_sort_workspace(n, num_experts);
   if (!workspace || workspace_bytes < need) return AOPS_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (n > 0 && n <= kSmallSort) {
+    moe_sort_small_kernel<<<1, kSmallSort, 0, s>>>(expert_ids, (int)n, (int)num_experts, sorted_idx,
+                                                  inverse_idx, group_list);
+    return record_launch_status(hipGetLastError());
+  }
   const int slices = (int)moe_slices(n);
   const int buckets = (int)num_experts + 1;
   int id_bits = 1;  // bits needed for bucket numbers 0..num_experts
