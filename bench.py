@@ -239,14 +239,18 @@ def bench_rope(L, ops, R, dev, cpu, B, config, note=None):
                  torch.get_num_threads(), note)
 
 
-def bench_reshape_and_cache(L, ops, R, dev, cpu, T, config, note=None):
+def bench_reshape_and_cache(L, ops, R, dev, cpu, T, config, note=None, consecutive=False):
     import torch
 
     Hkv, D, NB, P = 8, 128, 1024, 128
     torch.manual_seed(0)
     key = torch.randn(T, Hkv, D).half()
     value = torch.randn(T, Hkv, D).half()
-    slots = torch.randperm(NB * P)[:T].int()
+    if consecutive:  # a prefill: every sequence of 512 tokens fills four pages in order, the pages are scattered
+        pages = torch.randperm(NB)[: T // P]
+        slots = (pages[:, None] * P + torch.arange(P)[None, :]).reshape(-1).int()
+    else:
+        slots = torch.randperm(NB * P)[:T].int()
     alg = 4 * T * Hkv * D * 2 + T * 4
     n = n_sets_for(alg, lo=2, hi=48)
     n_cache = 2  # 2 x (2 x 256 MiB): a cache pair is reused only after 1 GiB of other lines
@@ -726,6 +730,9 @@ def main():
                            "scaled shape: shows the kernel's asymptotic bandwidth, not a BASELINE config"),
         bench_reshape_and_cache(L, ops, R, dev, False, 65536, "2 scaled x32: reshape_and_cache",
                                 "scaled shape: shows the kernel's asymptotic bandwidth, not a BASELINE config"),
+        bench_reshape_and_cache(L, ops, R, dev, False, 65536, "2 scaled x32, slots in page order: reshape_and_cache",
+                                "scaled shape with the slot pattern of a prefill (whole pages in token order, pages "
+                                "scattered) instead of BASELINE's random permutation", consecutive=True),
         bench_swiglu(L, ops, R, dev, False, 8192, 14336, "3 scaled x32: swiglu",
                      "scaled shape: shows the kernel's asymptotic bandwidth, not a BASELINE config"),
         bench_rope(L, ops, R, dev, False, 16384, "5 scaled x256: rope",
