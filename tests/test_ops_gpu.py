@@ -439,6 +439,45 @@ def test_dense_mlp_chain(ops, dev):
     torch.testing.assert_close(y.cpu().float(), R.mlp_ref(x, gu, dn).float(), **GMM_TOL)
 
 
+@pytest.mark.parametrize("pattern", ["prefill", "random", "mixed"])
+@pytest.mark.parametrize("with_value", [True, False])
+def test_reshape_and_cache_prefill_sized(ops, dev, pattern, with_value):
+    """Prefill-sized calls, bit-exact for the slot patterns a caller produces: whole pages in token order, a random
+    permutation, and a mix with a swapped pair, slots outside the cache, a run that crosses a page boundary and a
+    token count that is not a multiple of anything."""
+    g = _gen(31)
+    Hkv, D, NB, P = 8, 128, 96, 128
+    T = 4096 + (0 if pattern == "prefill" else 13)
+    assert (T + P - 1) // P <= NB // 2
+    key = torch.randn(T, Hkv, D, generator=g).half()
+    value = torch.randn(T, Hkv, D, generator=g).half()
+    if pattern == "random":
+        slots = torch.randperm(NB * P, generator=g)[:T].int()
+    else:
+        pages = 2 * torch.randperm(NB // 2, generator=g)[: (T + P - 1) // P]   # even pages: the odd ones stay free
+        slots = (pages[:, None] * P + torch.arange(P)[None, :]).reshape(-1)[:T].int()
+        if pattern == "mixed":
+            slots[40], slots[41] = slots[41].clone(), slots[40].clone()   # run broken inside a tile
+            slots[100] = -1                                                 # skipped token
+            slots[200] = NB * P                                             # outside the cache
+            slots[352:384] = slots[352:384] + 16                            # consecutive, but crossing into the next page
+    kc0 = torch.randn(NB, Hkv * D // 16, P, 16, generator=g).half()
+    vc0 = torch.randn(NB, Hkv * D // 16, P, 16, generator=g).half()
+    kcd, vcd = kc0.to(dev), vc0.to(dev)
+    kc_ref, vc_ref = kc0.clone(), vc0.clone()
+    if pattern == "mixed":  # duplicate targets would make the result depend on the write order: keep slots unique
+        valid = slots[(slots >= 0) & (slots < NB * P)]
+        assert valid.unique().numel() == valid.numel()
+    if with_value:
+        ops.reshape_and_cache(key.to(dev), value.to(dev), kcd, vcd, slots.to(dev))
+        R.reshape_and_cache_ref(key, kc_ref, slots, value, vc_ref)
+    else:
+        ops.reshape_and_cache(key.to(dev), None, kcd, None, slots.to(dev))
+        R.reshape_and_cache_ref(key, kc_ref, slots)
+    assert torch.equal(kcd.cpu(), kc_ref)
+    assert torch.equal(vcd.cpu(), vc_ref)
+
+
 # ----------------------------------------------------------------------------- paged attention
 def _paged_case(B, Hq, Hkv, D, P, lens, seed, max_pages=None, extra_pages=5, poison=False):
     g = _gen(seed)
