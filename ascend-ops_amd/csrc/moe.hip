@@ -248,12 +248,13 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-  // four routed rows at a time, loads first (independent), then the fp32 accumulation in the order of k
-  for (int k0 = 0; k0 < topk; k0 += 4) {
-    f16x8 v[4];
-    float wgt[4];
+  constexpr int kRows = 8;
+  // eight routed rows at a time, loads first (independent), then the fp32 accumulation in the order of k
+  for (int k0 = 0; k0 < topk; k0 += kRows) {
+    f16x8 v[kRows];
+    float wgt[kRows];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kRows; ++j) {
       const int k = k0 + j;
       const int64_t f = t * topk + (k < topk ? k : topk - 1);
       const int id = ids[f];
@@ -265,7 +266,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
       if (!ok) v[j] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < kRows; ++j)
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(wgt[j], (float)v[j][e], acc[e]);
   }
