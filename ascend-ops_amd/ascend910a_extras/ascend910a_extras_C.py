@@ -268,22 +268,13 @@ def matmul(x, w):
     return y
 
 
-def _few_rows_per_expert(rows: int, num_experts: int) -> bool:
-    """True for routed batches of decode size (under 48 rows per expert on average): the weights are then
-    streamed for little arithmetic, and the small-tile kernels of ``grouped_matmul`` followed by a separate
-    activation beat the fused kernel, whose work items are 320 rows tall."""
-    return rows < 48 * max(1, min(rows, num_experts))
-
-
 def grouped_matmul_swiglu(x, w, group_list):
-    """swiglu(grouped_matmul(x, w, group_list)) in one kernel where the fused kernel supports the
-    shape (K a multiple of 128, at least 256), as two kernels otherwise.  Not part of the
+    """swiglu(grouped_matmul(x, w, group_list)) in one kernel (the library picks the persistent kernel or,
+    for few rows per expert and for K that is not a multiple of 128, a small-tile one).  Not part of the
     reference's surface: it fuses the chain csrc/ffi/ops.cpp:157-233 -> 110-154 of an expert MLP."""
     _check_grouped_matmul("grouped_matmul_swiglu", x, w, group_list)
     num_tokens, dim = x.shape
     num_experts, inner_dim = w.size(0), w.size(2)
-    if dim % 128 != 0 or dim < 256 or _few_rows_per_expert(num_tokens, num_experts):
-        return swiglu(grouped_matmul(x, w, group_list))
     y = torch.empty((num_tokens, inner_dim // 2), dtype=x.dtype, device=x.device)
     code = _lib.aops_grouped_matmul_swiglu_f16(
         _ptr(x), _ptr(w), _ptr(group_list), _ptr(y), num_tokens, dim, num_experts, inner_dim, _stream(x.device)
@@ -509,7 +500,7 @@ def grouped_matmul_swiglu_gather(x, sorted_idx, topk, w, group_list):
            lambda: f"{name}: sorted_idx must have tokens*topk entries, got {sorted_idx.numel()} for {x.size(0)} tokens, topk {topk}")
     rows = sorted_idx.numel()
     dim = x.size(1)
-    if dim % 128 != 0 or dim < 256 or x.size(0) * dim >= 2 ** 32 or _few_rows_per_expert(rows, w.size(0)):
+    if x.size(0) * dim >= 2 ** 32:  # the kernel addresses the rows of x with 32-bit offsets
         return grouped_matmul_swiglu(moe_gather(x, sorted_idx, group_list, topk), w, group_list)
     # the remaining checks are those of grouped_matmul on the (virtual) gathered matrix
     _check(w.dim() == 3 and group_list.dim() == 1 and group_list.is_contiguous(), lambda: f"{name}: w must be 3D, group_list 1D")

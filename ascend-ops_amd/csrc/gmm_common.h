@@ -283,6 +283,12 @@ int gmm_launch_persistent(bool swiglu, const f16* x, const f16* w, const int64_t
                           int64_t rows, int k, int num_experts, int n, hipStream_t stream,
                           const int32_t* row_idx, int idx_div, int64_t x_rows);
 
+// Fused gate_up + SwiGLU (row_idx != nullptr: + row gather) on 128 x 128 tiles, or 64 x 64 with
+// `small`; k a multiple of 64.
+int gmm_launch_tiles_fused(bool small, const f16* x, const f16* w, const int64_t* group_list, f16* y,
+                           int64_t rows, int k, int num_experts, int n, hipStream_t stream,
+                           const int32_t* row_idx, int idx_div, int64_t x_rows);
+
 // Dense [m, k] x [n, k]^T with the k range split over several workgroups per output tile and a
 // second kernel adding the partial results: for few rows and a long k, where whole-k tiles would
 // leave most CUs without work.  gmm_splitk_workspace returns the bytes of fp32 scratch the call

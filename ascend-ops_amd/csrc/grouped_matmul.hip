@@ -80,11 +80,22 @@ extern "C" int aops_grouped_matmul_f16(const void* x, const void* w, const int64
   return aops_grouped_matmul_impl(x, w, group_list, y, rows, k, num_experts, n, stream);
 }
 
+// Kernel choice of the fused entry points: 0 = persistent 320 x 256 kernel, 1 = 128 x 128 tiles,
+// 2 = 64 x 64 tiles.  Under 96 rows per expert the weights are streamed for little arithmetic and the
+// small tiles win (see the tile choice above); the persistent kernel also needs k % 128 == 0, k >= 256.
+static int fused_tile_choice(int64_t rows, int64_t k, int64_t num_experts) {
+  const int64_t groups = num_experts < rows ? num_experts : rows;
+  const int64_t avg = groups > 0 ? (rows + groups - 1) / groups : 0;
+  if (k % 128 != 0 || k < 256) return avg < 24 ? 2 : 1;
+  if (avg >= 96) return 0;
+  return avg < 24 ? 2 : 1;
+}
+
 extern "C" int aops_grouped_matmul_swiglu_f16(const void* x, const void* w, const int64_t* group_list,
                                               void* y, int64_t rows, int64_t k, int64_t num_experts,
                                               int64_t n, void* stream) {
   using namespace aops;
-  if (rows < 0 || k <= 0 || n <= 0 || num_experts < 0 || k % 128 != 0 || k < 256 || n % 64 != 0)
+  if (rows < 0 || k <= 0 || n <= 0 || num_experts < 0 || k % 64 != 0 || n % 64 != 0)
     return AOPS_ERR_INVALID_ARGUMENT;
   // 32-bit per-lane offsets: (n/2 + 32) weight rows of k elements must fit
   if (rows > 0x7fffffff - 4096 || k > (1 << 22) || n > 0x7fffffff || num_experts > (1 << 20) ||
@@ -92,6 +103,11 @@ extern "C" int aops_grouped_matmul_swiglu_f16(const void* x, const void* w, cons
     return AOPS_ERR_INVALID_ARGUMENT;
   if (rows == 0 || num_experts == 0) return AOPS_OK;
   if (!x || !w || !group_list || !y) return AOPS_ERR_INVALID_ARGUMENT;
+  const int choice = fused_tile_choice(rows, k, num_experts);
+  if (choice != 0)
+    return gmm_launch_tiles_fused(choice == 2, static_cast<const f16*>(x), static_cast<const f16*>(w),
+                                  group_list, static_cast<f16*>(y), rows, (int)k, (int)num_experts, (int)n,
+                                  static_cast<hipStream_t>(stream), nullptr, 1, 1);
   return gmm_launch_persistent(true, static_cast<const f16*>(x), static_cast<const f16*>(w), group_list,
                                static_cast<f16*>(y), rows, (int)k, (int)num_experts, (int)n,
                                static_cast<hipStream_t>(stream), nullptr, 1, 1);
@@ -135,7 +151,7 @@ extern "C" int aops_grouped_matmul_swiglu_gather_f16(const void* x, const int32_
                                                      int64_t k, int64_t num_experts, int64_t n,
                                                      void* stream) {
   using namespace aops;
-  if (rows < 0 || k <= 0 || n <= 0 || num_experts < 0 || k % 128 != 0 || k < 256 || n % 64 != 0 ||
+  if (rows < 0 || k <= 0 || n <= 0 || num_experts < 0 || k % 64 != 0 || n % 64 != 0 ||
       idx_div <= 0 || idx_div > 0x7fffffff || x_rows < 0 || (rows > 0 && x_rows == 0))
     return AOPS_ERR_INVALID_ARGUMENT;
   // 32-bit per-lane offsets: x_rows activation rows and (n/2 + 32) weight rows of k elements must fit
@@ -144,6 +160,11 @@ extern "C" int aops_grouped_matmul_swiglu_gather_f16(const void* x, const int32_
     return AOPS_ERR_INVALID_ARGUMENT;
   if (rows == 0 || num_experts == 0) return AOPS_OK;
   if (!x || !row_idx || !w || !group_list || !y) return AOPS_ERR_INVALID_ARGUMENT;
+  const int choice = fused_tile_choice(rows, k, num_experts);
+  if (choice != 0)
+    return gmm_launch_tiles_fused(choice == 2, static_cast<const f16*>(x), static_cast<const f16*>(w),
+                                  group_list, static_cast<f16*>(y), rows, (int)k, (int)num_experts, (int)n,
+                                  static_cast<hipStream_t>(stream), row_idx, (int)idx_div, x_rows);
   return gmm_launch_persistent(true, static_cast<const f16*>(x), static_cast<const f16*>(w), group_list,
                                static_cast<f16*>(y), rows, (int)k, (int)num_experts, (int)n,
                                static_cast<hipStream_t>(stream), row_idx, (int)idx_div, x_rows);

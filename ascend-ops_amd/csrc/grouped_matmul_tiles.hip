@@ -16,12 +16,22 @@ namespace aops {
 //   global -> registers, D tiles ahead (the loads of tile kt+1+D are issued in iteration kt),
 //   registers -> LDS stage (kt+1)&1 during iteration kt, one barrier per k tile,
 //   LDS -> MFMA fragments one 16-wide k step ahead of the matrix cores.
-template <int MB, int NB, int D>
+//
+// SWIGLU = true fuses the activation of a gate_up projection: with d = n/2 the kernel writes
+// y[r, c] = silu(h[r, c]) * h[r, d + c] (h = x @ W_e^T) as a [rows, d] matrix.  A work item then
+// covers BN/2 output columns: the first half of its weight tile holds their gate rows, the second
+// half the up rows d further down, and the two meet in the LDS staging of the epilogue (after the
+// rounding to fp16, as in the two-kernel chain).  GATHER = true reads activation row j of the sorted
+// batch from row row_idx[j] / idx_div of x (see grouped_matmul_persistent_kernel).
+template <int MB, int NB, int D, bool SWIGLU = false, bool GATHER = false>
 __global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
     const f16* __restrict__ x, const f16* __restrict__ w, const int64_t* __restrict__ group_list,
-    f16* __restrict__ y, int64_t rows, int k, int num_experts, int n) {
+    f16* __restrict__ y, int64_t rows, int k, int num_experts, int n,
+    const int32_t* __restrict__ row_idx, int idx_div, uint32_t x_rows) {
   constexpr int BM = 64 * MB;
   constexpr int BN = 64 * NB;
+  constexpr int BNO = SWIGLU ? BN / 2 : BN;  // output columns per work item
+  const int n_out = SWIGLU ? n / 2 : n;      // output row length
   constexpr int kThreads = 4 * kWave;
   constexpr int kAChunks = BM * (kBK / 8) / kThreads;  // 16-byte chunks per thread and tile
   constexpr int kBChunks = BN * (kBK / 8) / kThreads;
@@ -34,7 +44,7 @@ __global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
   f16* sa = smem;                 // [2][BM * kBK]
   f16* sb = smem + 2 * BM * kBK;  // [2][BN * kBK]
 
-  const int n_tiles = (n + BN - 1) / BN;
+  const int n_tiles = (n_out + BNO - 1) / BNO;
   const GmmWork work =
       gmm_find_work<BM>(group_list, num_experts, rows, n_tiles, blockIdx.x, gridDim.x);
   if (!work.valid) return;
@@ -54,21 +64,35 @@ __global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
   // one per-lane offset plus compile-time strides.
   const int ld_row = tid >> 3;
   const int ld_kc = tid & 7;
-  const f16* a_base = x + (int64_t)work.row_begin * k;
-  const f16* b_base = w + ((int64_t)work.expert * n + (int64_t)work.n_tile * BN) * k;
+  const f16* a_base = GATHER ? x : x + (int64_t)work.row_begin * k;
+  const f16* b_base = w + ((int64_t)work.expert * n + (int64_t)work.n_tile * BNO) * k;
   uint32_t a_off[kAChunks], b_off[kBChunks];
-  const int n_left = n - work.n_tile * BN;  // rows of w available to this tile (>= 64)
+  const int n_left = n_out - work.n_tile * BNO;  // output columns available to this tile (>= 32)
 #pragma unroll
   for (int i = 0; i < kAChunks; ++i) {
     int ar = ld_row + kRowsPerPass * i;
     if (ar > tile_rows - 1) ar = tile_rows - 1;  // rows past the group: duplicates, never stored
-    a_off[i] = (uint32_t)ar * (uint32_t)k + ld_kc * 8;
+    if constexpr (GATHER) {
+      uint32_t src = (uint32_t)row_idx[work.row_begin + ar] / (uint32_t)idx_div;
+      src = src < x_rows ? src : x_rows - 1;  // an index outside x reads its last row instead of faulting
+      a_off[i] = src * (uint32_t)k + ld_kc * 8;
+    } else {
+      a_off[i] = (uint32_t)ar * (uint32_t)k + ld_kc * 8;
+    }
   }
 #pragma unroll
   for (int i = 0; i < kBChunks; ++i) {
     int br = ld_row + kRowsPerPass * i;
-    if (br > n_left - 1) br = n_left - 1;  // n is a multiple of 64, not necessarily of BN
-    b_off[i] = (uint32_t)br * (uint32_t)k + ld_kc * 8;
+    if constexpr (SWIGLU) {
+      // tile rows [0, BN/2): gate rows of the item's columns; [BN/2, BN): the up rows n_out further down
+      const bool up = br >= BN / 2;
+      int c = up ? br - BN / 2 : br;
+      if (c > n_left - 1) c = n_left - 1;
+      b_off[i] = (uint32_t)(c + (up ? n_out : 0)) * (uint32_t)k + ld_kc * 8;
+    } else {
+      if (br > n_left - 1) br = n_left - 1;  // n is a multiple of 64, not necessarily of BN
+      b_off[i] = (uint32_t)br * (uint32_t)k + ld_kc * 8;
+    }
   }
   const int st_dst = lds_off(ld_row, ld_kc);
 
@@ -235,6 +259,28 @@ __global__ __launch_bounds__(4 * kWave) void grouped_matmul_kernel(
     }
   }
   __syncthreads();
+  if constexpr (SWIGLU) {
+    constexpr int kChunksPerRow = BNO / 8;  // 16-byte chunks per output row of the tile
+    constexpr int kRowsPerStorePass = kThreads / kChunksPerRow;
+    const int c16 = tid % kChunksPerRow;
+    const int col = work.n_tile * BNO + c16 * 8;
+    if (col < n_out) {
+      for (int m = tid / kChunksPerRow; m < tile_rows; m += kRowsPerStorePass) {
+        const f16x8 gv = *reinterpret_cast<const f16x8*>(&sc[m * BN + ((c16 ^ (m & kSwz)) << 3)]);
+        const f16x8 uv =
+            *reinterpret_cast<const f16x8*>(&sc[m * BN + (((c16 + kChunksPerRow) ^ (m & kSwz)) << 3)]);
+        f16x8 v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float gf = (float)gv[e];
+          const float ex = __builtin_amdgcn_exp2f(-1.4426950408889634f * gf);
+          v[e] = (f16)(gf * (float)uv[e] * __builtin_amdgcn_rcpf(1.0f + ex));
+        }
+        st128(y + (int64_t)(work.row_begin + m) * n_out + col, v);
+      }
+    }
+    return;
+  }
   constexpr int kChunksPerRow = BN / 8;              // 16-byte chunks per tile row
   constexpr int kRowsPerStorePass = kThreads / kChunksPerRow;
   const int c16 = tid % kChunksPerRow;
@@ -729,21 +775,24 @@ int gmm_launch_splitk(const f16* x, const f16* w, f16* y, float* workspace, size
   return record_launch_status(hipGetLastError());
 }
 
-template <int MB, int NB, int D>
+template <int MB, int NB, int D, bool SWIGLU = false, bool GATHER = false>
 static int gmm_launch(const f16* x, const f16* w, const int64_t* group_list, f16* y, int64_t rows,
-                      int k, int num_experts, int n, hipStream_t stream) {
+                      int k, int num_experts, int n, hipStream_t stream,
+                      const int32_t* row_idx = nullptr, int idx_div = 1, int64_t x_rows = 1) {
   constexpr int BM = 64 * MB;
   constexpr int BN = 64 * NB;
   constexpr int kStageBytes = 2 * (BM + BN) * kBK * (int)sizeof(f16);
   constexpr int kTileBytes = BM * BN * (int)sizeof(f16);
   constexpr int kLds = kStageBytes > kTileBytes ? kStageBytes : kTileBytes;
   static_assert(kLds <= 160 * 1024, "LDS budget");
-  const int64_t n_tiles = (n + BN - 1) / BN;
+  constexpr int BNO = SWIGLU ? BN / 2 : BN;
+  const int64_t n_out = SWIGLU ? n / 2 : n;
+  const int64_t n_tiles = (n_out + BNO - 1) / BNO;
   const int64_t max_m_tiles = (rows + BM - 1) / BM + num_experts;
   int64_t grid = max_m_tiles * n_tiles;
   grid = (grid + kXcds - 1) / kXcds * kXcds;
   if (grid > 0x7fffffff) return AOPS_ERR_INVALID_ARGUMENT;
-  auto kernel = grouped_matmul_kernel<MB, NB, D>;
+  auto kernel = grouped_matmul_kernel<MB, NB, D, SWIGLU, GATHER>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -751,7 +800,8 @@ static int gmm_launch(const f16* x, const f16* w, const int64_t* group_list, f16
     if (e != hipSuccess) return record_launch_status(e);
     attr_set = true;
   }
-  kernel<<<(unsigned)grid, 4 * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts, n);
+  kernel<<<(unsigned)grid, 4 * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts, n, row_idx,
+                                                       idx_div, (uint32_t)x_rows);
   return record_launch_status(hipGetLastError());
 }
 
@@ -775,6 +825,22 @@ int gmm_launch_tiles(int variant, const f16* x, const f16* w, const int64_t* gro
     default:  // 64 x 64 tiles
       return gmm_launch<1, 1, 2>(x, w, group_list, y, rows, k, num_experts, n, stream);
   }
+}
+
+// The fused gate_up + SwiGLU (+ row gather) on the small tiles, for batches with few rows per expert:
+// 128 x 128 tiles (64 output columns per item) or 64 x 64 (32 output columns).
+int gmm_launch_tiles_fused(bool small, const f16* x, const f16* w, const int64_t* group_list, f16* y,
+                           int64_t rows, int k, int num_experts, int n, hipStream_t stream,
+                           const int32_t* row_idx, int idx_div, int64_t x_rows) {
+  if (row_idx) {
+    if (small)
+      return gmm_launch<1, 1, 2, true, true>(x, w, group_list, y, rows, k, num_experts, n, stream, row_idx,
+                                             idx_div, x_rows);
+    return gmm_launch<2, 2, 2, true, true>(x, w, group_list, y, rows, k, num_experts, n, stream, row_idx,
+                                           idx_div, x_rows);
+  }
+  if (small) return gmm_launch<1, 1, 2, true>(x, w, group_list, y, rows, k, num_experts, n, stream);
+  return gmm_launch<2, 2, 2, true>(x, w, group_list, y, rows, k, num_experts, n, stream);
 }
 
 }  // namespace aops

@@ -167,10 +167,12 @@ int aops_matmul_nt_ws_f16(const void* x, const void* w, void* y, void* workspace
  * Grouped matmul of a gate_up projection with the SwiGLU activation fused into its epilogue:
  *   h = x[rows of expert e] (fp32 accumulate) @ w[e]^T          (never stored)
  *   y[r, c] = f16( silu(h[r, c]) * h[r, n/2 + c] ),  c < n/2
- * x, w, group_list as for aops_grouped_matmul_f16; y: [rows, n/2].  Equal, up to the fp16 rounding
- * of h that it skips, to aops_grouped_matmul_f16 followed by aops_swiglu_f16, without the
- * [rows, n] intermediate.  k must be a multiple of 128 and at least 256, n a multiple of 64;
- * other shapes return AOPS_ERR_INVALID_ARGUMENT (call the two operators instead).
+ * x, w, group_list as for aops_grouped_matmul_f16 (k and n multiples of 64); y: [rows, n/2].
+ * Equal, within fp16 rounding, to aops_grouped_matmul_f16 followed by aops_swiglu_f16, without
+ * the [rows, n] intermediate.  Large routed batches (48 rows per expert and more, k a multiple of
+ * 128 from 256 on) run the persistent 320 x 256 kernel, which applies the activation to the fp32
+ * accumulators; fewer rows per expert or another k run small tiles, which round h to fp16 first,
+ * as the two-operator chain does.
  * Replaces the chain aclnnGroupedMatMulEx -> aclnnSwiGluEx of an expert MLP (reference
  * csrc/ffi/ops.cpp:211-218 and 138-145, chained as in benchmark/test_mlp.py:37-41); the reference
  * has no fused operator.

@@ -93,11 +93,11 @@ def test_c_abi_rejects_bad_sizes_without_touching_the_gpu():
     assert lib.aops_matmul_nt_workspace(16, 100, 64) == 0                                   # invalid shape: no workspace
     assert lib.aops_grouped_matmul_f16(ctypes.c_void_p(8), ctypes.c_void_p(8), None, ctypes.c_void_p(8), 4, 64, 1, 64, None) == -1
     # fused extensions
-    assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 192, 2, 128, None) == -1   # k % 128
-    assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 128, 2, 128, None) == -1   # k < 256
+    assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 160, 2, 128, None) == -1   # k % 64
+    assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 128, 2, 96, None) == -1    # n % 64
     assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 256, 2, 128, None) == -1   # null pointers
     assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 0, 256, 2, 128, None) == 0
-    assert lib.aops_grouped_matmul_swiglu_gather_f16(None, None, 8, 16, None, None, None, 128, 192, 2, 128, None) == -1  # k % 128
+    assert lib.aops_grouped_matmul_swiglu_gather_f16(None, None, 8, 16, None, None, None, 128, 160, 2, 128, None) == -1  # k % 64
     assert lib.aops_grouped_matmul_swiglu_gather_f16(None, None, 0, 16, None, None, None, 128, 256, 2, 128, None) == -1  # divisor
     assert lib.aops_grouped_matmul_swiglu_gather_f16(None, None, 8, 16, None, None, None, 128, 256, 2, 128, None) == -1  # null pointers
     assert lib.aops_grouped_matmul_swiglu_gather_f16(None, None, 8, 16, None, None, None, 0, 256, 2, 128, None) == 0

@@ -339,7 +339,9 @@ def test_grouped_matmul_every_kernel(ops, dev, monkeypatch, variant, rows, K, N,
         (1300, 256, 192, 6, [0, 1, 700, 0, 330, 200]),   # ragged groups, N/2 = 96 (three column blocks of the last tile)
         (4096, 512, 1536, 64, None),                      # several work items per workgroup
         (700, 2048, 1536, 1, [650]),                      # one expert, rows past the group untouched
-        (300, 192, 128, 3, [100, 100, 100]),              # K not a multiple of 128: two-kernel path
+        (300, 192, 128, 3, [100, 100, 100]),              # K not a multiple of 128: the small-tile fused kernel
+        (90, 256, 192, 20, None),                         # few rows per expert: 64 x 64 tiles, 96 output columns
+        (1200, 512, 320, 30, None),                       # 40 rows per expert: 128 x 128 tiles, ragged last column tile
     ],
 )
 def test_grouped_matmul_swiglu_fused(ops, dev, rows, K, N, E, counts):
