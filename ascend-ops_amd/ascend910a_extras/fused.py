@@ -10,7 +10,8 @@ import ascend910a_extras.ascend910a_extras_C as _C
 def grouped_matmul_swiglu(x: torch.Tensor, w: torch.Tensor, group_list: torch.Tensor) -> torch.Tensor:
     """``ops.swiglu(ops.grouped_matmul(x, w, group_list))`` without the ``[rows, N]`` intermediate:
     the gate_up projection of an expert MLP (reference ``benchmark/test_mlp.py:37-41``) with the
-    activation applied to the fp32 accumulators.  Returns ``[rows, N/2]``."""
+    activation applied in the matmul's epilogue (to the fp32 accumulators in the large-batch kernel, to
+    the fp16-rounded product in the small-tile kernels).  Returns ``[rows, N/2]``."""
     return _C.grouped_matmul_swiglu(x, w, group_list)
 
 
