@@ -395,7 +395,7 @@ def _gmm_swiglu_gather_entry(L, dev, w_storage, tokens, topk):
                  "extension: replaces moe_gather + gate_up + swiglu; one weight set, so the weights are re-read from HBM every launch but x (17 MB) stays cached")
 
 
-def _moe_mlp_entry(dev, w1_storage, w2_storage, tokens, topk):
+def _moe_mlp_entry(dev, w1_storage, w2_storage, tokens, topk, decode=False):
     """The whole routed expert MLP of configs[3] through the extension API (sort -> gate_up with gather and SwiGLU
     -> down -> combine), captured in one HIP graph: what the operators add up to for a caller."""
     import torch
@@ -423,6 +423,17 @@ def _moe_mlp_entry(dev, w1_storage, w2_storage, tokens, topk):
         trials.append(_events_ms(graph.replay, 10) * 1e3 / 10)
     trials.sort()
     flops = 2 * tokens * topk * K * N1 + 2 * tokens * topk * (N1 // 2) * K
+    if decode:
+        # a decode step: the weights of every expert that is hit are streamed once, the arithmetic is negligible
+        hit = int(torch.unique(ids).numel())
+        wbytes = hit * (N1 * K + K * (N1 // 2)) * 2
+        e = {"op": "moe_mlp", "config": f"4 at decode size ({tokens} tokens): routed expert MLP end to end (extension)",
+             "shape": f"x [{tokens},{K}], top-{topk} of {E} experts ({hit} hit), inter {N1 // 2}", "bound": "hbm",
+             "algorithmic_bytes": wbytes, "gpu_us": round(trials[len(trials) // 2], 3), "gpu_us_min": round(trials[0], 3)}
+        e["GBps"] = round(wbytes / e["gpu_us"] / 1e3, 1)
+        e["hbm_frac"] = round(e["GBps"] / HBM_PEAK_GBPS, 4)
+        e["note"] = "weight-stream bound: bytes = the fp16 weights of the experts that are hit"
+        return e
     e = {"op": "moe_mlp", "config": "4: routed expert MLP end to end (extension, five launches in one graph)",
          "shape": f"x [{tokens},{K}], top-{topk} of {E} experts, inter {N1 // 2}", "bound": "mfma",
          "algorithmic_flops": flops, "gpu_us": round(trials[len(trials) // 2], 3), "gpu_us_min": round(trials[0], 3)}
@@ -491,6 +502,7 @@ def bench_moe(L, ops, R, dev, cpu):
     e_fused = _gmm_swiglu_entry(L, ops, dev, "4: MoE gate_up + activation, fused", x, w1, gl, h_dev)
     e_gather = _gmm_swiglu_gather_entry(L, dev, w1, tokens, topk)
     e_layer = _moe_mlp_entry(dev, w1, w2, tokens, topk)
+    e_decode = _moe_mlp_entry(dev, w1, w2, 64, topk, decode=True)
     del w1
     h = ops.swiglu(h_dev)
     # swiglu at the MoE shape
@@ -512,6 +524,7 @@ def bench_moe(L, ops, R, dev, cpu):
     out.append(e_fused)
     out.append(e_gather)
     out.append(e_layer)
+    out.append(e_decode)
     out.extend(_moe_glue_entries(L, dev, E, hidden, tokens, topk))
     tot_flops = e1["algorithmic_flops"] + e2["algorithmic_flops"]
     tot_us = e1["gpu_us"] + e2["gpu_us"]
