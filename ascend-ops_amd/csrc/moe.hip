@@ -276,44 +276,88 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(
   st128_stream(out + (t * vec_per_row + c) * 8, o);
 }
 
-// Routing tables of a few tokens (at most kSmallSort ids): one workgroup, one launch.  Thread t
-// ranks id t by counting the ids that sort in front of it (smaller bucket, or the same bucket and
-// a smaller index: stable), thread e counts the ids of experts 0..e for group_list; both walk the
-// buckets held in LDS.
-constexpr int kSmallSort = 128;  // quadratic work on one CU: beyond this the sliced sort is faster
+// Routing tables of a decode step (at most kSmallSort ids): one workgroup, one launch.  Histogram
+// with LDS atomics, exclusive scan of the buckets by all four waves (group_list falls out of it),
+// then wave 0 walks the ids in order, 64 at a time, exactly as moe_scatter_kernel walks a slice.
+constexpr int kSmallSort = 1024;
+constexpr int kSmallThreads = 4 * kWave;
+constexpr int kSmallPerThread = (kMoeMaxExperts + 1) / kSmallThreads;  // consecutive buckets per thread in the scan
 
-__global__ __launch_bounds__(kSmallSort) void moe_sort_small_kernel(
+__global__ __launch_bounds__(kSmallThreads) void moe_sort_small_kernel(
     const int32_t* __restrict__ ids, int n, int num_experts, int32_t* __restrict__ sorted_idx,
-    int32_t* __restrict__ inverse_idx, int64_t* __restrict__ group_list) {
-  __shared__ __attribute__((aligned(16))) int32_t bucket[kSmallSort];
+    int32_t* __restrict__ inverse_idx, int id_bits, int64_t* __restrict__ group_list) {
+  __shared__ int32_t bucket[kSmallSort];
+  __shared__ int32_t running[kMoeMaxExperts + 1];
+  __shared__ int32_t wave_total[4];
   const int t = threadIdx.x;
-  // entries past n hold a bucket larger than any real one: they are never counted
-  const int mine = t < n ? moe_bucket(ids[t], num_experts) : num_experts + 1;
-  bucket[t] = mine;
-  __syncthreads();
-  const int n4 = (n + 3) / 4;
-  const int4* b4 = reinterpret_cast<const int4*>(bucket);
-  if (t < n) {
-    int rank = 0;
-#pragma unroll 8
-    for (int j = 0; j < n4; ++j) {  // same address in every lane: one LDS broadcast per four ids
-      const int4 o = b4[j];
-      rank += (o.x < mine || (o.x == mine && 4 * j < t)) ? 1 : 0;
-      rank += (o.y < mine || (o.y == mine && 4 * j + 1 < t)) ? 1 : 0;
-      rank += (o.z < mine || (o.z == mine && 4 * j + 2 < t)) ? 1 : 0;
-      rank += (o.w < mine || (o.w == mine && 4 * j + 3 < t)) ? 1 : 0;
-    }
-    sorted_idx[rank] = t;
-    if (inverse_idx) inverse_idx[t] = rank;
+  const int lane = t & (kWave - 1);
+  const int wave = t / kWave;
+  const int buckets = num_experts + 1;
+  for (int e = t; e < kMoeMaxExperts + 1; e += kSmallThreads) running[e] = 0;
+  int mine[kSmallSort / kSmallThreads];
+#pragma unroll
+  for (int u = 0; u < kSmallSort / kSmallThreads; ++u) {
+    const int i = t + u * kSmallThreads;
+    mine[u] = i < n ? moe_bucket(ids[i], num_experts) : buckets;
   }
-  for (int e = t; e < num_experts; e += kSmallSort) {
-    int upto = 0;
-#pragma unroll 8
-    for (int j = 0; j < n4; ++j) {
-      const int4 o = b4[j];
-      upto += (o.x <= e ? 1 : 0) + (o.y <= e ? 1 : 0) + (o.z <= e ? 1 : 0) + (o.w <= e ? 1 : 0);
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < kSmallSort / kSmallThreads; ++u) {
+    const int i = t + u * kSmallThreads;
+    bucket[i] = mine[u];
+    if (i < n) atomicAdd(&running[mine[u]], 1);
+  }
+  __syncthreads();
+  // exclusive scan: thread t owns buckets [t*kSmallPerThread, (t+1)*kSmallPerThread)
+  int cnt[kSmallPerThread];
+  int sum = 0;
+#pragma unroll
+  for (int u = 0; u < kSmallPerThread; ++u) {
+    cnt[u] = running[t * kSmallPerThread + u];
+    sum += cnt[u];
+  }
+  int incl = sum;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int up = __shfl_up(incl, d);
+    if (lane >= d) incl += up;
+  }
+  if (lane == kWave - 1) wave_total[wave] = incl;
+  __syncthreads();
+  int excl = incl - sum;
+  for (int v = 0; v < wave; ++v) excl += wave_total[v];
+#pragma unroll
+  for (int u = 0; u < kSmallPerThread; ++u) {
+    const int e = t * kSmallPerThread + u;
+    running[e] = excl;
+    excl += cnt[u];
+    if (e < num_experts) group_list[e] = excl;
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  for (int i0 = 0; i0 < n; i0 += kWave) {
+    const int i = i0 + lane;
+    const bool live = i < n;
+    const int e = live ? bucket[i] : 0;
+    uint64_t same = __ballot(live);
+    for (int bit = 0; bit < id_bits; ++bit) {
+      const bool set = (e >> bit) & 1;
+      const uint64_t m = __ballot(set);
+      same &= set ? m : ~m;
     }
-    group_list[e] = upto;
+    const int leader = live ? __builtin_ctzll(same) : lane;
+    int first = 0;
+    if (live && lane == leader) {
+      first = running[e];
+      running[e] = first + __builtin_popcountll(same);
+    }
+    first = __shfl(first, leader);
+    if (live) {
+      const int pos = first + __builtin_popcountll(same & lt_mask);
+      sorted_idx[pos] = i;
+      if (inverse_idx) inverse_idx[i] = pos;
+    }
   }
 }
 
@@ -338,15 +382,16 @@ extern "C" int aops_moe_sort_i32(const int32_t* expert_ids, int64_t n, int64_t n
   const size_t need = aops_moe_sort_workspace(n, num_experts);
   if (!workspace || workspace_bytes < need) return AOPS_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (n > 0 && n <= kSmallSort) {
-    moe_sort_small_kernel<<<1, kSmallSort, 0, s>>>(expert_ids, (int)n, (int)num_experts, sorted_idx,
-                                                  inverse_idx, group_list);
+  int id_bits = 1;  // bits needed for bucket numbers 0..num_experts
+  while ((1 << id_bits) <= (int)num_experts) ++id_bits;
+  // one launch instead of two up to 512 ids, instead of three (more than 256 buckets) up to 1024
+  if (n > 0 && (n <= kSmallSort / 2 || (n <= kSmallSort && num_experts + 1 > kFoldBuckets))) {
+    moe_sort_small_kernel<<<1, kSmallThreads, 0, s>>>(expert_ids, (int)n, (int)num_experts, sorted_idx,
+                                                     inverse_idx, id_bits, group_list);
     return record_launch_status(hipGetLastError());
   }
   const int slices = (int)moe_slices(n);
   const int buckets = (int)num_experts + 1;
-  int id_bits = 1;  // bits needed for bucket numbers 0..num_experts
-  while ((1 << id_bits) <= (int)num_experts) ++id_bits;
   int32_t* counts = static_cast<int32_t*>(workspace);           // [slices][E+1]
   int32_t* base = counts + (int64_t)slices * buckets;           // [E+1]
   const size_t lds = (size_t)kMoeWaves * buckets * sizeof(int32_t);

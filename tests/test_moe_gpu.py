@@ -16,9 +16,11 @@ H = torch.float16
         (4096, 8, 128, False),     # configs[3] routing
         (1000, 2, 8, True),        # n not a multiple of the slice, ids -1 and E mixed in
         (1, 1, 1, False),
-        (16, 8, 128, True),        # 128 ids: the largest table of the one-launch sort
-        (129, 1, 128, True),       # one id more: the sliced sort
+        (128, 8, 128, True),       # 1024 ids: the largest table of the one-workgroup sort
+        (205, 5, 128, True),       # 1025 ids: the sliced sort
         (8, 8, 4095, False),
+        (100, 8, 4095, True),
+        (63, 1, 2, False),
         (77, 6, 300, True),        # more experts than lanes of a wave
         (513, 1, 4095, False),     # largest expert count
         (20000, 4, 3, False),      # long runs of equal ids
