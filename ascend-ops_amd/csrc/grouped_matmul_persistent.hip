@@ -389,13 +389,43 @@ static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* grou
   return record_launch_status(hipGetLastError());
 }
 
+// Tile height of the persistent kernel: 320 rows (one tile covers a typical expert of a large routed
+// batch) or 256 rows when that takes fewer rounds of work items over the CUs times rows per tile - the
+// wall time of a compute-bound product.  group_list stays on the device, so the groups are taken as
+// equal plus two standard deviations of a uniform routing; a single group is exact.
+static bool gmm_prefer_256_rows(int64_t rows, int64_t num_experts, int64_t n_out_tiles, int cus) {
+  const int64_t groups = num_experts < rows ? num_experts : rows;
+  if (groups <= 0) return false;
+  int64_t avg = (rows + groups - 1) / groups;
+  if (groups > 1) {
+    int64_t sd = 1;
+    while (sd * sd < avg) ++sd;
+    avg += 2 * sd;
+  }
+  auto cost = [&](int64_t bm) {
+    const int64_t items = groups * ((avg + bm - 1) / bm) * n_out_tiles;
+    return ((items + cus - 1) / cus) * bm;
+  };
+  return cost(256) < cost(320);
+}
+
 int gmm_launch_persistent(bool swiglu, const f16* x, const f16* w, const int64_t* group_list, f16* y,
                           int64_t rows, int k, int num_experts, int n, hipStream_t stream,
                           const int32_t* row_idx, int idx_div, int64_t x_rows) {
-  if (row_idx)  // only the fused gate_up form gathers
+  const int64_t n_out_tiles = swiglu ? (n / 2 + 127) / 128 : (n + 255) / 256;
+  const bool small = gmm_prefer_256_rows(rows, num_experts, n_out_tiles, 256);
+  if (row_idx) {  // only the fused gate_up form gathers
+    if (small)
+      return gmm_persistent_launch<4, 2, 4, true, true>(x, w, group_list, y, rows, k, num_experts, n, stream,
+                                                        row_idx, idx_div, x_rows);
     return gmm_persistent_launch<5, 2, 4, true, true>(x, w, group_list, y, rows, k, num_experts, n, stream,
                                                       row_idx, idx_div, x_rows);
-  if (swiglu) return gmm_persistent_launch<5, 2, 4, true>(x, w, group_list, y, rows, k, num_experts, n, stream);
+  }
+  if (swiglu) {
+    if (small) return gmm_persistent_launch<4, 2, 4, true>(x, w, group_list, y, rows, k, num_experts, n, stream);
+    return gmm_persistent_launch<5, 2, 4, true>(x, w, group_list, y, rows, k, num_experts, n, stream);
+  }
+  if (small) return gmm_persistent_launch<4, 2, 4, false>(x, w, group_list, y, rows, k, num_experts, n, stream);
   return gmm_persistent_launch<5, 2, 4, false>(x, w, group_list, y, rows, k, num_experts, n, stream);
 }
 

@@ -427,6 +427,30 @@ def test_matmul_nt_ws_without_split(ops, dev):
     assert torch.equal(a, b)
 
 
+def test_persistent_kernel_with_256_row_tiles(ops, dev):
+    """8192 rows in one group and 2048 columns: 256-row tiles cover the rows in 32 work items per column tile where
+    320-row tiles would need 26 with the last one mostly empty, so the library takes the 256-row form of the
+    persistent kernel - plain, with the fused activation, and with the row gather."""
+    import ascend910a_extras.ascend910a_extras_C as C
+    import ascend910a_extras.fused as fused
+    g = _gen(41)
+    rows, K, N = 8192, 256, 2048
+    x = torch.randn(rows, K, generator=g).half()
+    w = (torch.randn(1, N, K, generator=g) / K ** 0.5).half().transpose(1, 2)
+    gl = torch.tensor([rows - 100], dtype=torch.int64)
+    xd, wd, gd = x.to(dev), w.to(dev), gl.to(dev)
+    end = int(gl[-1])
+    ref = x.float() @ w[0].float()
+    y = ops.grouped_matmul(xd, wd, gd)
+    torch.testing.assert_close(y[:end].cpu().float(), ref[:end], **GMM_TOL)
+    act = fused.grouped_matmul_swiglu(xd, wd, gd)
+    act_ref = (torch.nn.functional.silu(ref[:, : N // 2]) * ref[:, N // 2:])
+    torch.testing.assert_close(act[:end].cpu().float(), act_ref[:end], **GMM_TOL)
+    perm = torch.randperm(rows, generator=g).int()
+    gathered = C.grouped_matmul_swiglu_gather(xd, perm.to(dev), 1, wd, gd)
+    assert torch.equal(gathered[:end], fused.grouped_matmul_swiglu(xd[perm.long().to(dev)], wd, gd)[:end])
+
+
 def test_dense_mlp_chain(ops, dev):
     """benchmark/test_mlp.py:37-41 through grouped_matmul with one expert (reduced width)."""
     g = _gen(0)
