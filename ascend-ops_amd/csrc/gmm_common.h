@@ -24,6 +24,22 @@ __device__ __forceinline__ int64_t gmm_group_end(const int64_t* __restrict__ gro
   return group_list ? group_list[e] : rows;
 }
 
+// Order of the work items of one expert with t m-tiles and n_tiles n-tiles: bands of kBandM m-tiles;
+// inside a band the m-tiles of one weight tile are adjacent and the weight tiles follow one another.
+// Workgroups that run side by side then share a weight tile among up to kBandM of them and an
+// activation tile among n_tiles / ... of them (a 2-d block of the output instead of a column), which
+// keeps more of the operand traffic inside the XCD's L2.  With t <= kBandM (routed batches) this is the
+// plain "m-tiles of a weight tile adjacent" order.
+constexpr int kBandM = 8;
+__device__ __forceinline__ void gmm_item_to_tile(int local, int t, int n_tiles, int& m_tile, int& n_tile) {
+  const int per_band = kBandM * n_tiles;
+  const int band = local / per_band;
+  const int r = local - band * per_band;
+  const int m_in_band = min(kBandM, t - band * kBandM);
+  n_tile = r / m_in_band;
+  m_tile = band * kBandM + (r - n_tile * m_in_band);
+}
+
 struct GmmWork {
   int expert;
   int row_begin;  // first row of this m-tile
@@ -90,8 +106,9 @@ __device__ __forceinline__ GmmWork gmm_find_work(const int64_t* __restrict__ gro
       if (work < base + span) {
         const int local = (int)(work - base);
         f_expert = e;
-        f_ntile = local / t;  // m-tiles of one weight tile are adjacent
-        f_begin = prev + (local - f_ntile * t) * kBM;
+        int m_tile;
+        gmm_item_to_tile(local, t, n_tiles, m_tile, f_ntile);
+        f_begin = prev + m_tile * kBM;
         f_end = end;
         break;
       }
@@ -231,8 +248,9 @@ __device__ __forceinline__ GmmWork gmm_locate(const GmmPlan& p,
         if (!found && t > 0 && work < base + span) {
           const int local = (int)(work - base);
           f_expert = e0 + j;
-          f_ntile = local / t;
-          f_begin = prev + (local - f_ntile * t) * kBM;
+          int m_tile;
+          gmm_item_to_tile(local, t, n_tiles, m_tile, f_ntile);
+          f_begin = prev + m_tile * kBM;
           f_end = end;
           found = true;
         }
@@ -250,8 +268,9 @@ __device__ __forceinline__ GmmWork gmm_locate(const GmmPlan& p,
         if (work < base + span) {
           const int local = (int)(work - base);
           f_expert = e;
-          f_ntile = local / t;
-          f_begin = prev + (local - f_ntile * t) * kBM;
+          int m_tile;
+          gmm_item_to_tile(local, t, n_tiles, m_tile, f_ntile);
+          f_begin = prev + m_tile * kBM;
           f_end = end;
           break;
         }
