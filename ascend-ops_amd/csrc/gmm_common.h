@@ -26,10 +26,10 @@ __device__ __forceinline__ int64_t gmm_group_end(const int64_t* __restrict__ gro
 
 // Order of the work items of one expert with t m-tiles and n_tiles n-tiles: bands of kBandM m-tiles;
 // inside a band the m-tiles of one weight tile are adjacent and the weight tiles follow one another.
-// Workgroups that run side by side then share a weight tile among up to kBandM of them and an
-// activation tile among n_tiles / ... of them (a 2-d block of the output instead of a column), which
-// keeps more of the operand traffic inside the XCD's L2.  With t <= kBandM (routed batches) this is the
-// plain "m-tiles of a weight tile adjacent" order.
+// The 32 workgroups that run side by side on an XCD then cover a 2-d block of the output (kBandM
+// m-tiles x 32 / kBandM weight tiles) instead of one column of it and find most of both operands in
+// that XCD's L2.  With t <= kBandM (routed batches) this is the plain "m-tiles of a weight tile
+// adjacent" order.
 constexpr int kBandM = 8;
 __device__ __forceinline__ void gmm_item_to_tile(int local, int t, int n_tiles, int& m_tile, int& n_tile) {
   const int per_band = kBandM * n_tiles;
