@@ -53,3 +53,20 @@ def test_no_kernel_reads_a_matrix_core_result_early(tmp_path):
         found = scanner.scan(text)
         assert not found, f"{path.name}: matrix-core results read too early: {found[:5]}"
     assert total_mfma > 1000, "the scan must have seen the matrix-core kernels"
+
+
+def test_no_packed_fp32_instructions(tmp_path):
+    """The library is built with packed fp32 arithmetic switched off (-packed-fp32-ops): no kernel may contain
+    v_pk_add_f32, v_pk_mul_f32 or v_pk_fma_f32."""
+    import re
+
+    spec = importlib.util.spec_from_file_location("aops_build", os.path.join(ROOT, "ascend-ops_amd", "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    kernels = 0
+    for path in build.emit_assembly(tmp_path):
+        text = path.read_text()
+        kernels += text.count(".amdhsa_kernel ")
+        found = sorted(set(re.findall(r"v_pk_(?:add|mul|fma)_f32", text)))
+        assert not found, f"{path.name}: packed fp32 instructions {found}"
+    assert kernels > 50, "the check must have seen the library's kernels"
