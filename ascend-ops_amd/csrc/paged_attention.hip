@@ -81,7 +81,11 @@ static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_si
     return e ? atoi(e) : -1;
   }();
   constexpr int64_t kCus = 256;
-  if (!forced && balanced_env != 0 && bs <= kWave && bs * num_kv_heads < 2 * kCus && max_units >= 2) {
+  // ... and whenever the block table allows contexts beyond 4096 tokens: whole sequences per workgroup
+  // would let one long sequence among short ones occupy eight CUs for the whole launch.
+  constexpr int64_t kSkewFreeLen = 4096;
+  if (!forced && balanced_env != 0 && bs <= kWave && max_units >= 2 &&
+      (bs * num_kv_heads < 2 * kCus || max_len > kSkewFreeLen || balanced_env > 0)) {
     const int64_t total = balanced_env > 0 ? balanced_env : kCus;
     int64_t wgs = (total + num_kv_heads - 1) / num_kv_heads;
     if (wgs > bs * max_units) wgs = bs * max_units;  // never more shares than units
