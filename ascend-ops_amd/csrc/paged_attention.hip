@@ -49,6 +49,12 @@ struct PaChunking {
 
 constexpr int kPaUnit = kPaWaves * kPaStep;  // 256 tokens: one step of every wave
 
+// Batches of up to kPaPlanMax sequences can use the balanced partition; above 64 sequences it is
+// computed by a one-workgroup kernel into kPaPlanInts(bs) ints behind the partial results.
+constexpr int64_t kPaPlanMax = 4096;
+constexpr int64_t kPaMaxShares = 256;
+static size_t pa_tail_ints(int64_t bs) { return bs <= 64 ? (size_t)bs : (size_t)(2 * bs + 1 + kPaMaxShares); }
+
 static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_size,
                               int64_t max_blocks_per_seq) {
   const int64_t max_len = block_size * max_blocks_per_seq;
@@ -84,10 +90,11 @@ static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_si
   // ... and whenever the block table allows contexts beyond 4096 tokens: whole sequences per workgroup
   // would let one long sequence among short ones occupy eight CUs for the whole launch.
   constexpr int64_t kSkewFreeLen = 4096;
-  if (!forced && balanced_env != 0 && bs <= kWave && max_units >= 2 &&
+  if (!forced && balanced_env != 0 && bs <= kPaPlanMax && max_units >= 2 &&
       (bs * num_kv_heads < 2 * kCus || max_len > kSkewFreeLen || balanced_env > 0)) {
     const int64_t total = balanced_env > 0 ? balanced_env : kCus;
     int64_t wgs = (total + num_kv_heads - 1) / num_kv_heads;
+    if (wgs > kPaMaxShares) wgs = kPaMaxShares;
     if (wgs > bs * max_units) wgs = bs * max_units;  // never more shares than units
     c.balanced_wgs = (int)wgs;
     c.max_splits = (int)(wgs < max_units ? wgs : max_units);
@@ -432,18 +439,98 @@ __device__ __forceinline__ int pa_share_of(int x, int wgs, int total) {
   return (int)((((int64_t)x + 1) * wgs - 1) / total);
 }
 
+// The same partition for batches of more than 64 sequences, computed once by one workgroup into
+//   plan[0] = total units, plan[1 + b] = units in front of sequence b, plan[1 + bs + b] = its clamped
+//   length, plan[1 + 2*bs + w] = the sequence that holds the first unit of share w.
+constexpr int kPaPlanThreads = 1024;
+
+__global__ __launch_bounds__(kPaPlanThreads) void pa_plan_kernel(const int32_t* __restrict__ context_lens,
+                                                                 int bs, int max_len, int wgs_max,
+                                                                 int32_t* __restrict__ plan) {
+  __shared__ int wave_sum[kPaPlanThreads / kWave];
+  __shared__ int carry_s;
+  const int t = threadIdx.x;
+  const int lane = t & (kWave - 1);
+  const int wave = t / kWave;
+  if (t == 0) carry_s = 0;
+  __syncthreads();
+  for (int b0 = 0; b0 < bs; b0 += kPaPlanThreads) {
+    const int b = b0 + t;
+    const int len = b < bs ? min(max(context_lens[b], 0), max_len) : 0;
+    const int units = (len + kPaUnit - 1) / kPaUnit;
+    int incl = units;
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+      const int up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    if (lane == kWave - 1) wave_sum[wave] = incl;
+    __syncthreads();
+    int before = carry_s + incl - units;
+    for (int v = 0; v < wave; ++v) before += wave_sum[v];
+    if (b < bs) {
+      plan[1 + b] = before;
+      plan[1 + bs + b] = len;
+    }
+    __syncthreads();
+    if (t == kPaPlanThreads - 1) carry_s = before + units;
+    __syncthreads();
+  }
+  const int total = carry_s;
+  if (t == 0) plan[0] = total;
+  if (total == 0) return;
+  // every sequence names itself as the start of the shares whose first unit it holds
+  const int wgs = min(wgs_max, total);
+  for (int b = t; b < bs; b += kPaPlanThreads) {
+    const int before = plan[1 + b];  // written by this thread
+    const int units = (plan[1 + bs + b] + kPaUnit - 1) / kPaUnit;
+    if (units == 0) continue;
+    // shares w with before <= floor(w * total / wgs) < before + units
+    int w = (int)(((int64_t)before * wgs + total - 1) / total);
+    for (; w < wgs && (int)((int64_t)w * total / wgs) < before + units; ++w) plan[1 + 2 * bs + w] = b;
+  }
+}
+
 // grid = (wgs, Hkv), block = 8 waves.  Workgroup w walks through its share of the batch's units,
 // sequence by sequence; the part of sequence b it covers becomes partial result number
-// w - (share holding b's first unit) of that sequence.
+// w - (share holding b's first unit) of that sequence.  plan == nullptr: at most 64 sequences, the
+// partition is computed by every wave (pa_units); otherwise it is read from pa_plan_kernel's output.
 template <int D, int GMAX>
 __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_balanced(
     const f16* __restrict__ q, const f16* __restrict__ key_cache,
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ context_lens, float* __restrict__ part_o,
     float* __restrict__ part_ml, int bs, int num_kv_heads, int block_size, int max_blocks_per_seq,
-    int max_splits, float scale_log2, int num_blocks, int group) {
+    int max_splits, float scale_log2, int num_blocks, int group, const int32_t* __restrict__ plan) {
   const int w = blockIdx.x;
   const int g = blockIdx.y;
+  if (plan) {
+    const int total = plan[0];
+    const int wgs = min((int)gridDim.x, total);
+    if (w >= wgs) return;
+    const int lo = (int)((int64_t)w * total / wgs);
+    const int hi = (int)((int64_t)(w + 1) * total / wgs);
+    int cur = lo;
+    int b = plan[1 + 2 * bs + w];
+    while (cur < hi && b < bs) {
+      const int before = plan[1 + b];
+      const int len = plan[1 + bs + b];
+      const int units = (len + kPaUnit - 1) / kPaUnit;
+      if (units > 0) {
+        const int seg_end = min(hi, before + units);
+        const int tok0 = (cur - before) * kPaUnit;
+        const int tok1 = min((seg_end - before) * kPaUnit, len);
+        const int slot = w - pa_share_of(before, wgs, total);
+        pa_process_chunk<D, GMAX, false>(q, key_cache, value_cache, block_tables, part_o, part_ml, nullptr, b, g,
+                                         len, tok0, tok1 - tok0, slot, num_kv_heads, block_size,
+                                         max_blocks_per_seq, max_splits, scale_log2, num_blocks, group);
+        cur = seg_end;
+        if (cur < hi) __syncthreads();  // the LDS arrays of the chunk are reused
+      }
+      ++b;
+    }
+    return;
+  }
   const PaUnits pu = pa_units(context_lens, bs, max_blocks_per_seq * block_size);
   // no more shares than units: every share then holds at least one unit, and the shares of a
   // sequence are consecutive
@@ -479,7 +566,7 @@ __global__ __launch_bounds__(kPaD) void pa_decode_merge(const float* __restrict_
                                                         const int32_t* __restrict__ context_lens,
                                                         f16* __restrict__ o, int num_heads,
                                                         int chunk_tokens, int max_splits, int balanced_wgs,
-                                                        int bs, int max_len) {
+                                                        int bs, int max_len, const int32_t* __restrict__ plan) {
   const int h = blockIdx.x;
   const int b = blockIdx.y;
   const int d = threadIdx.x;
@@ -490,7 +577,13 @@ __global__ __launch_bounds__(kPaD) void pa_decode_merge(const float* __restrict_
     return;
   }
   int nsplit;
-  if (balanced_wgs > 0) {  // partial results of the shares that hold the sequence's first and last unit
+  if (balanced_wgs > 0 && plan) {
+    const int total = plan[0];
+    const int before = plan[1 + b];
+    const int units = (plan[1 + bs + b] + kPaUnit - 1) / kPaUnit;
+    const int wgs = min(balanced_wgs, total);
+    nsplit = pa_share_of(before + units - 1, wgs, total) - pa_share_of(before, wgs, total) + 1;
+  } else if (balanced_wgs > 0) {  // partial results of the shares that hold the sequence's first and last unit
     const PaUnits pu = pa_units(context_lens, bs, max_len);
     const int before = __builtin_amdgcn_readlane(pu.before, b);
     const int units = __builtin_amdgcn_readlane(pu.units, b);
@@ -519,14 +612,19 @@ static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t*
                       PaChunking ch, hipStream_t s, int num_blocks, int32_t* order) {
   const float scale_log2 = kLog2e / __builtin_sqrtf((float)kPaD);
   if (ch.balanced_wgs > 0) {
+    const int32_t* plan = nullptr;
+    if (bs > kWave) {  // `order` is the int area behind the partial results
+      pa_plan_kernel<<<1, kPaPlanThreads, 0, s>>>(cl, bs, max_blocks_per_seq * block_size, ch.balanced_wgs, order);
+      plan = order;
+    }
     dim3 bgrid((unsigned)ch.balanced_wgs, (unsigned)num_kv_heads);
     pa_decode_balanced<kPaD, GMAX><<<bgrid, kPaWaves * kWave, 0, s>>>(
         q, kc, vc, bt, cl, part_o, part_ml, bs, num_kv_heads, block_size, max_blocks_per_seq,
-        ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads);
+        ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads, plan);
     dim3 mgrid((unsigned)num_heads, (unsigned)bs);
     pa_decode_merge<kPaD><<<mgrid, kPaD, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
                                            ch.max_splits, ch.balanced_wgs, bs,
-                                           max_blocks_per_seq * block_size);
+                                           max_blocks_per_seq * block_size, plan);
     return;
   }
   dim3 grid((unsigned)ch.max_splits, (unsigned)num_kv_heads, (unsigned)bs);
@@ -543,7 +641,7 @@ static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t*
       ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads, order);
   dim3 mgrid((unsigned)num_heads, (unsigned)bs);
   pa_decode_merge<kPaD><<<mgrid, kPaD, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
-                                         ch.max_splits, 0, bs, max_blocks_per_seq * block_size);
+                                         ch.max_splits, 0, bs, max_blocks_per_seq * block_size, nullptr);
 }
 
 // Generic path for every other shape (head_dim a multiple of 16 up to 256, any block size, any
@@ -651,9 +749,9 @@ extern "C" size_t aops_paged_attention_workspace(int64_t bs, int64_t num_heads,
     return 0;
   if (!pa_fast_shape(num_heads, num_kv_heads, head_dim, block_size)) return 16;  // not used
   const PaChunking ch = pa_chunking(bs, num_kv_heads, block_size, max_blocks_per_seq);
-  // partial results, then one int per sequence (the length order of batches above 64 sequences)
+  // partial results, then the ints of the length order or of the balanced partition's plan
   return (size_t)bs * (size_t)num_heads * (size_t)ch.max_splits * (size_t)(head_dim + 2) * sizeof(float) +
-         (size_t)bs * sizeof(int32_t);
+         pa_tail_ints(bs) * sizeof(int32_t);
 }
 
 extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,

@@ -670,13 +670,16 @@ def test_paged_attention_matrix_core_path_other_head_sizes(ops, dev, B, Hq, Hkv,
         (33, 16, 4, 16, 700, 4),       # 16-token pages
         (12, 32, 8, 128, 255, 5),      # every sequence shorter than one 256-token unit
         (64, 32, 8, 128, 9000, 6),     # 512 pairs, but a block table wide enough for one long sequence among short ones
+        (130, 32, 8, 128, 9000, 7),    # more than 64 sequences: the partition comes from a one-workgroup plan kernel
+        (1100, 2, 1, 64, 4500, 8),     # more sequences than the plan kernel has threads
     ],
 )
 def test_paged_attention_balanced_partition(ops, dev, B, Hq, Hkv, P, maxlen, seed):
     """Batches with fewer than two (sequence, kv head) pairs per CU, or whose block table allows contexts beyond 4096
     tokens: the token stream is cut into equal shares of 256-token units, one per workgroup, whatever the sequence
     boundaries; a share may hold the end of one sequence, whole sequences and the start of another.  Empty sequences
-    in between, NaN in unused slots."""
+    in between, NaN in unused slots.  Up to 64 sequences every wave derives the partition itself; above that a
+    one-workgroup kernel writes it into the workspace first."""
     import random
     rnd = random.Random(seed)
     lens = [rnd.choice([0, 1, 255, 256, 257, rnd.randint(1, maxlen), rnd.randint(1, maxlen)]) for _ in range(B)]
