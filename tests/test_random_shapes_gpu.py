@@ -43,6 +43,39 @@ def test_paged_attention_random_shape(ops, dev, seed):
     torch.testing.assert_close(o.float(), ref.float(), **TOL)
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_paged_attention_random_batch(ops, dev, seed):
+    """Batch sizes on either side of every switch of the launcher (a wave's 64 lanes, the ranking kernel, the plan
+    kernel of the balanced partition), short sequences with a few long ones among them, tables wider than needed."""
+    rnd = random.Random(100 + seed)
+    g = torch.Generator().manual_seed(100 + seed)
+    D = rnd.choice([64, 128, 128, 256])
+    P = rnd.choice([16, 64, 128])
+    Hkv = rnd.choice([1, 2, 8])
+    Hq = Hkv * rnd.choice([1, 4])
+    B = rnd.choice([rnd.randint(2, 20), rnd.randint(60, 70), rnd.randint(100, 300)])
+    long_len = rnd.choice([700, 3000, 5000])
+    lens = [rnd.choice([0, 1, 255, 256, 257, rnd.randint(1, 300)]) for _ in range(B)]
+    for _ in range(rnd.randint(1, 3)):
+        lens[rnd.randrange(B)] = rnd.randint(long_len // 2, long_len)
+    pages_per = [(l + P - 1) // P for l in lens]
+    max_pages = max(pages_per) + rnd.choice([0, 1, 40])
+    NB = sum(pages_per) + 3
+    perm = torch.randperm(NB, generator=g)
+    bt = torch.full((B, max_pages), -1, dtype=torch.int32)
+    c = 0
+    for b, n in enumerate(pages_per):
+        bt[b, :n] = perm[c:c + n].int()
+        c += n
+    kc = R.nz_pack(torch.randn(NB, P, Hkv, D, generator=g).half())
+    vc = R.nz_pack(torch.randn(NB, P, Hkv, D, generator=g).half())
+    q = torch.randn(B, Hq, D, generator=g).half()
+    cl = torch.tensor(lens, dtype=torch.int32)
+    o = ops.paged_attention(q.to(dev), kc.to(dev), vc.to(dev), bt.to(dev), cl.to(dev)).cpu()
+    ref = R.paged_attention_ref(q, kc, vc, bt.clamp(min=0), cl)
+    torch.testing.assert_close(o.float(), ref.float(), **TOL)
+
+
 @pytest.mark.parametrize("seed", range(8))
 def test_token_operators_random_shape(ops, dev, seed):
     rnd = random.Random(100 + seed)
