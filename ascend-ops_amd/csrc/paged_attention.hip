@@ -52,6 +52,7 @@ constexpr int kPaUnit = kPaWaves * kPaStep;  // 256 tokens: one step of every wa
 // Batches of up to kPaPlanMax sequences can use the balanced partition; above 64 sequences it is
 // computed by a one-workgroup kernel into kPaPlanInts(bs) ints behind the partial results.
 constexpr int64_t kPaPlanMax = 4096;
+constexpr int64_t kPaMaxChunks = 512;  // partial results per (sequence, head) at most
 constexpr int64_t kPaMaxShares = 256;
 static size_t pa_tail_ints(int64_t bs) { return bs <= 64 ? (size_t)bs : (size_t)(2 * bs + 1 + kPaMaxShares); }
 
@@ -74,6 +75,8 @@ static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_si
     return (v >= kPaWaves * kPaStep && v % (kPaWaves * kPaStep) == 0) ? v : 0;
   }();
   if (forced) chunk = forced;
+  if ((max_len + chunk - 1) / chunk > kPaMaxChunks)  // the merge kernel keeps one weight per chunk in LDS
+    chunk = (int)(((max_units + kPaMaxChunks - 1) / kPaMaxChunks) * kUnit);
   PaChunking c;
   c.chunk_tokens = chunk;
   c.max_splits = (int)((max_len + chunk - 1) / chunk);
@@ -559,21 +562,29 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_balanced(
   }
 }
 
-// grid = (Hq, bs), block = head_dim: one thread per output element.
+// grid = (Hq, bs), block = 4 waves.  Every wave works out the weights 2^(m_s - max m) of the partial
+// results (a lane per result); wave v then adds up the results s = v, v+4, ... with eight row loads in
+// flight (a lane holds head_dim/64 neighbouring output elements), and the four sums meet in LDS.
+constexpr int kPaMergeWaves = 4;
+constexpr int kPaMergeMaxSplits = (int)kPaMaxChunks;  // weights kept in LDS; pa_chunking never cuts a sequence finer
+
 template <int kPaD>
-__global__ __launch_bounds__(kPaD) void pa_decode_merge(const float* __restrict__ part_o,
-                                                        const float* __restrict__ part_ml,
-                                                        const int32_t* __restrict__ context_lens,
-                                                        f16* __restrict__ o, int num_heads,
-                                                        int chunk_tokens, int max_splits, int balanced_wgs,
-                                                        int bs, int max_len, const int32_t* __restrict__ plan) {
+__global__ __launch_bounds__(kPaMergeWaves* kWave) void pa_decode_merge(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml,
+    const int32_t* __restrict__ context_lens, f16* __restrict__ o, int num_heads, int chunk_tokens,
+    int max_splits, int balanced_wgs, int bs, int max_len, const int32_t* __restrict__ plan) {
+  constexpr int kPer = kPaD / kWave;  // output elements per lane
+  typedef float fvec __attribute__((ext_vector_type(kPer)));
+  __shared__ float wts[kPaMergeMaxSplits];
+  __shared__ float red[kPaMergeWaves][kPaD];
   const int h = blockIdx.x;
   const int b = blockIdx.y;
-  const int d = threadIdx.x;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
   const int context_len = context_lens[b];
-  const int64_t out = ((int64_t)b * num_heads + h) * kPaD + d;
+  const int64_t out = ((int64_t)b * num_heads + h) * kPaD;
   if (context_len <= 0) {
-    o[out] = (f16)0.f;
+    if (threadIdx.x < kPaD) o[out + threadIdx.x] = (f16)0.f;
     return;
   }
   int nsplit;
@@ -592,17 +603,66 @@ __global__ __launch_bounds__(kPaD) void pa_decode_merge(const float* __restrict_
   } else {
     nsplit = (context_len + chunk_tokens - 1) / chunk_tokens;
   }
-  if (nsplit > max_splits) nsplit = max_splits;
+  nsplit = min(nsplit, min(max_splits, kPaMergeMaxSplits));
   const int64_t base = ((int64_t)b * num_heads + h) * max_splits;
+
+  // weights: the same in every wave; wave 0 leaves them in LDS
+  constexpr int kMlPerLane = kPaMergeMaxSplits / kWave;
+  float m_s[kMlPerLane], l_s[kMlPerLane];
   float mx = kNegBig;
-  for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, part_ml[(base + s) * 2]);
-  float lsum = 0.f, a = 0.f;
-  for (int s = 0; s < nsplit; ++s) {
-    const float wt = __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - mx);
-    lsum += part_ml[(base + s) * 2 + 1] * wt;
-    a += part_o[(base + s) * kPaD + d] * wt;
+#pragma unroll
+  for (int i = 0; i < kMlPerLane; ++i) {
+    const int s = i * kWave + lane;
+    m_s[i] = kNegBig;
+    l_s[i] = 0.f;
+    if (i * kWave < nsplit && s < nsplit) {  // first test is wave uniform: whole rounds are skipped
+      const float2 ml = *reinterpret_cast<const float2*>(&part_ml[(base + s) * 2]);
+      m_s[i] = ml.x;
+      l_s[i] = ml.y;
+    }
+    mx = fmaxf(mx, m_s[i]);
   }
-  o[out] = (f16)(lsum > 0.f ? a / lsum : 0.f);
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+  float lsum = 0.f;
+#pragma unroll
+  for (int i = 0; i < kMlPerLane; ++i) {
+    const int s = i * kWave + lane;
+    const float wt = s < nsplit ? __builtin_amdgcn_exp2f(m_s[i] - mx) : 0.f;
+    lsum += l_s[i] * wt;
+    if (wave == 0 && i * kWave < nsplit) wts[s] = wt;
+  }
+  lsum = wave_sum(lsum);
+  __syncthreads();
+
+  fvec acc;
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) acc[e] = 0.f;
+  constexpr int kInFlight = 8;
+  for (int s0 = wave; s0 < nsplit; s0 += kPaMergeWaves * kInFlight) {
+    fvec v[kInFlight];
+    float wt[kInFlight];
+#pragma unroll
+    for (int j = 0; j < kInFlight; ++j) {
+      const int s = s0 + j * kPaMergeWaves;
+      const int sc = min(s, nsplit - 1);  // past the end: a valid row with weight 0
+      v[j] = *reinterpret_cast<const fvec*>(&part_o[(base + sc) * kPaD + lane * kPer]);
+      wt[j] = s < nsplit ? wts[sc] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < kInFlight; ++j)
+#pragma unroll
+      for (int e = 0; e < kPer; ++e) acc[e] += v[j][e] * wt[j];  // fixed order: the result is deterministic
+  }
+#pragma unroll
+  for (int e = 0; e < kPer; ++e) red[wave][lane * kPer + e] = acc[e];
+  __syncthreads();
+  if (threadIdx.x < kPaD) {
+    float a = 0.f;
+#pragma unroll
+    for (int v = 0; v < kPaMergeWaves; ++v) a += red[v][threadIdx.x];
+    o[out + threadIdx.x] = (f16)(lsum > 0.f ? a / lsum : 0.f);
+  }
 }
 
 template <int kPaD, int GMAX>
@@ -622,7 +682,7 @@ static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t*
         q, kc, vc, bt, cl, part_o, part_ml, bs, num_kv_heads, block_size, max_blocks_per_seq,
         ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads, plan);
     dim3 mgrid((unsigned)num_heads, (unsigned)bs);
-    pa_decode_merge<kPaD><<<mgrid, kPaD, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
+    pa_decode_merge<kPaD><<<mgrid, kPaMergeWaves * kWave, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
                                            ch.max_splits, ch.balanced_wgs, bs,
                                            max_blocks_per_seq * block_size, plan);
     return;
@@ -640,7 +700,7 @@ static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t*
       q, kc, vc, bt, cl, part_o, part_ml, o, num_kv_heads, block_size, max_blocks_per_seq,
       ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads, order);
   dim3 mgrid((unsigned)num_heads, (unsigned)bs);
-  pa_decode_merge<kPaD><<<mgrid, kPaD, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
+  pa_decode_merge<kPaD><<<mgrid, kPaMergeWaves * kWave, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
                                          ch.max_splits, 0, bs, max_blocks_per_seq * block_size, nullptr);
 }
 
