@@ -8,7 +8,10 @@
  * device data on the host, so all of them can be captured into a HIP graph.
  * Return value: AOPS_OK (0) or a negative AOPS_ERR_* code; nothing is thrown
  * across this boundary.  All fp tensors are IEEE binary16 ("f16"), densely
- * packed and row-major in the shapes stated.
+ * packed and row-major in the shapes stated.  Every tensor and workspace
+ * pointer must be 16-byte aligned (the kernels move 128 bits per lane); any
+ * hipMalloc'ed buffer and any row of a tensor whose row length the operator
+ * accepts is.
  *
  * Each declaration names the reference interface it replaces: the two-phase
  * aclnn*GetWorkspaceSize / aclnn* pair that csrc/ffi/ops.cpp of the reference
