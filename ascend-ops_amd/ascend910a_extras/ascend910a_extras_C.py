@@ -124,7 +124,13 @@ def _stream(device: torch.device) -> int:
 
 
 def _ptr(t: torch.Tensor):
-    return t.data_ptr() if t.numel() > 0 else None
+    """Device address of ``t`` (None for an empty tensor); the kernels move 128 bits per lane."""
+    if t.numel() == 0:
+        return None
+    p = t.data_ptr()
+    if p & 15 and t.dtype == torch.float16:  # index tensors are read element by element
+        raise RuntimeError("fp16 tensor data must be 16-byte aligned (a view that starts inside a row is not)")
+    return p
 
 
 def rope(q, k, position_ids, cos_cache, sin_cache):

@@ -167,6 +167,20 @@ def test_argument_checks_follow_the_reference(ops):
     _raises(ops.swiglu, torch.zeros(4, 128, dtype=torch.float32), match="float16")
 
 
+def test_misaligned_fp16_views_are_refused():
+    """The kernels move 128 bits per lane: a contiguous view that starts 8 bytes into a row is refused by the
+    pointer helper every operator passes its tensors through; index tensors may start anywhere."""
+    import ascend910a_extras.ascend910a_extras_C as C
+
+    flat = torch.zeros(4 * 64 + 4, dtype=H)
+    assert C._ptr(flat[:256].view(4, 64)) == flat.data_ptr()
+    with pytest.raises(RuntimeError, match="16-byte aligned"):
+        C._ptr(flat[4:260].view(4, 64))
+    ids = torch.zeros(9, dtype=torch.int32)
+    assert C._ptr(ids[1:]) == ids.data_ptr() + 4
+    assert C._ptr(flat[:0]) is None
+
+
 def test_product_package_does_not_import_the_oracle():
     pkg = os.path.join(ROOT, "ascend-ops_amd")
     for dirpath, _, files in os.walk(pkg):
