@@ -70,6 +70,19 @@ __device__ __forceinline__ void rope_rotate8(const f16x8& x1, const f16x8& x2, c
   }
 }
 
+// Workgroups are dealt to the eight XCDs (each with its own L2) round robin by their index.  Where
+// neighbouring pieces of work write into the same 128-byte cache lines (tokens in neighbouring slots of
+// a paged cache), a line written from two XCDs reaches memory as two partial writes.  This renumbering
+// gives the workgroups with the same index mod 8 (same XCD) kRun consecutive pieces of work inside
+// every run of 8 * kRun workgroups; the incomplete run at the end of the grid keeps its order.
+template <uint32_t kRun>
+__device__ __forceinline__ uint32_t xcd_run_index(uint32_t wg, uint32_t num_wgs) {
+  static_assert((kRun & (kRun - 1)) == 0, "power of two");
+  constexpr uint32_t kSpan = 8u * kRun;
+  if (wg >= (num_wgs & ~(kSpan - 1u))) return wg;
+  return (wg & ~(kSpan - 1u)) + (wg & 7u) * kRun + ((wg >> 3) & (kRun - 1u));
+}
+
 // Launch-status bookkeeping shared by the host launchers.
 int record_launch_status(hipError_t e);
 

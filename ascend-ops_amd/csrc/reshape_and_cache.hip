@@ -14,7 +14,9 @@ __global__ __launch_bounds__(256) void reshape_and_cache_kernel(
     const f16* __restrict__ key, const f16* __restrict__ value, f16* __restrict__ key_cache,
     f16* __restrict__ value_cache, const int32_t* __restrict__ slot_indices, uint32_t total,
     uint32_t pieces_per_row, uint32_t block_size, int64_t num_slots) {
-  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  // neighbouring tokens on one XCD: 32 workgroups = 64 tokens at 1024 halfs per row
+  const uint32_t wg = xcd_run_index<32>(blockIdx.x, gridDim.x);
+  const uint32_t i = wg * 256u + threadIdx.x;
   if (i >= total) return;
   const uint32_t token = i / pieces_per_row;
   const uint32_t piece = i - token * pieces_per_row;  // 16-byte piece of the row

@@ -27,7 +27,8 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(
     const int32_t* __restrict__ slot_indices, uint32_t total, uint32_t per_token,
     uint32_t rope_threads, uint32_t num_heads, uint32_t num_kv_heads, uint32_t head_dim,
     uint32_t block_size, int64_t num_slots) {
-  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  // neighbouring tokens (whose cache slots share cache lines in a prefill) on one XCD
+  const uint32_t i = xcd_run_index<32>(blockIdx.x, gridDim.x) * 256u + threadIdx.x;
   if (i >= total) return;
   const uint32_t b = i / per_token;
   const uint32_t t = i - b * per_token;

@@ -169,7 +169,8 @@ def test_reshape_and_cache_skips_bad_slots_and_roundtrips(ops, dev):
     assert torch.count_nonzero(got) == 0
 
 
-@pytest.mark.parametrize("B,Hq,Hkv,D,NB,P", [(64, 32, 8, 128, 2304, 128), (5, 6, 2, 64, 7, 16), (3, 1, 1, 16, 4, 8), (17, 16, 16, 256, 9, 32)])
+@pytest.mark.parametrize("B,Hq,Hkv,D,NB,P", [(64, 32, 8, 128, 2304, 128), (5, 6, 2, 64, 7, 16), (3, 1, 1, 16, 4, 8), (17, 16, 16, 256, 9, 32),
+                                             (700, 8, 2, 128, 16, 64)])   # prefill-sized: more than 256 workgroups
 def test_rope_reshape_and_cache_fused_equals_the_chain(ops, dev, B, Hq, Hkv, D, NB, P):
     """One launch against rope -> reshape_and_cache: q, k and both caches bit for bit, including a slot that is
     out of range (skipped by both) and cache contents that must stay untouched; and against the oracle."""
@@ -204,7 +205,8 @@ def test_rope_reshape_and_cache_fused_equals_the_chain(ops, dev, B, Hq, Hkv, D, 
     assert torch.equal(kc_b.cpu(), kc_ref) and torch.equal(vc_b.cpu(), vc_ref)
 
 
-@pytest.mark.parametrize("B,Hq,Hkv,D,NB,P", [(64, 32, 8, 128, 2304, 128), (5, 6, 2, 64, 7, 16), (3, 1, 1, 16, 4, 8), (9, 4, 4, 256, 9, 32), (7, 3, 1, 32, 5, 4)])
+@pytest.mark.parametrize("B,Hq,Hkv,D,NB,P", [(64, 32, 8, 128, 2304, 128), (5, 6, 2, 64, 7, 16), (3, 1, 1, 16, 4, 8), (9, 4, 4, 256, 9, 32), (7, 3, 1, 32, 5, 4),
+                                             (1200, 4, 4, 64, 80, 16)])
 def test_qknorm_rope_reshape_and_cache_fused(ops, dev, B, Hq, Hkv, D, NB, P):
     """Per-head RMSNorm of q and k + rope + cache write in one launch, against the oracle (RMSNorm rounded to fp16,
     then rotated) and against the chain of separate device operators where those take the shape."""
