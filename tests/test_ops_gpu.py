@@ -696,6 +696,16 @@ def test_paged_attention_balanced_partition(ops, dev, B, Hq, Hkv, P, maxlen, see
     assert torch.equal(_run_pa(ops, dev, case), o)
 
 
+def test_paged_attention_very_long_context(ops, dev):
+    """Contexts of 200000 and 70000 tokens next to one of 5: 782 units of 256 tokens cut into 128 shares per kv
+    head, more than 100 partial results for the longest sequence."""
+    case = _paged_case(3, 8, 2, 128, 128, [200000, 70000, 5], seed=21)
+    o = _run_pa(ops, dev, case)
+    ref = R.paged_attention_ref(*case)
+    torch.testing.assert_close(o.float(), ref.float(), **TOL)
+    assert (o.float() - ref.float()).abs().max() < 3e-3
+
+
 def test_paged_attention_ignores_garbage_and_unused_table_entries(ops, dev):
     lens = [5, 130, 257, 1]
     clean = _paged_case(4, 32, 8, 128, 128, lens, seed=1, max_pages=6)
