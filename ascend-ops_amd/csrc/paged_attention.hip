@@ -130,16 +130,32 @@ struct PaState {
 
 // S^T[token][head] = K . Q^T, scaled to log2 units; lane (head n, kg) gets tokens
 // 16*(e/4) + 4kg + e%4, e = 0..7, of the step.
-template <int NS>
-__device__ __forceinline__ void pa_scores(const PaRegs<NS>& k, const f16x8 (&qreg)[NS],
-                                          float scale_log2, float (&sc)[8]) {
+// QLDS: the Q^T fragments are read from LDS (q_lds = this lane's slice, fragment s 512 halfs further)
+// instead of being held in registers: at head_dim 256 they would push the kernel into scratch.
+template <int NS, bool QLDS>
+__device__ __forceinline__ void pa_scores(const PaRegs<NS>& k, const f16x8 (&qreg)[QLDS ? 1 : NS],
+                                          const f16* q_lds, float scale_log2, float (&sc)[8]) {
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
   f32x4 sacc[2] = {zero4, zero4};
+  if constexpr (QLDS) {
+    // the empty asm hides that the address is the same in every step, so the fragments are not
+    // hoisted out of the token loop into registers
+    uint32_t off = 0;
+    asm volatile("" : "+v"(off));
 #pragma unroll
-  for (int g = 0; g < 2; ++g)
+    for (int s = 0; s < NS; ++s) {
+      const f16x8 qs = *reinterpret_cast<const f16x8*>(q_lds + off + s * (kWave * 8));
 #pragma unroll
-    for (int s = 0; s < NS; ++s)
-      sacc[g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(k[g][s], qreg[s], sacc[g], 0, 0, 0);
+      for (int g = 0; g < 2; ++g)
+        sacc[g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(k[g][s], qs, sacc[g], 0, 0, 0);
+    }
+  } else {
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+      for (int s = 0; s < NS; ++s)
+        sacc[g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(k[g][s], qreg[s], sacc[g], 0, 0, 0);
+  }
   // A matrix-core result may only be read six wait states after its instruction (four passes plus
   // two).  The compiler keeps that distance inside a basic block, but when it places the
   // accumulators in AGPRs and a taken branch (the "no further step" case of the caller) lies between
@@ -227,12 +243,24 @@ __device__ __forceinline__ void pa_process_chunk(
   const int num_heads = num_kv_heads * group;
 
   // Q^T operand: lane (head n, kg) holds q[head n][32s + 8kg ..+7]; heads >= group are zero rows.
-  f16x8 qreg[NS];
+  constexpr bool QLDS = NS > 4;
+  f16x8 qreg[QLDS ? 1 : NS];
+  __shared__ __attribute__((aligned(16))) f16 sm_q[QLDS ? NS * kWave * 8 : 8];
+  const f16* q_lds = sm_q + lane * 8;
   {
     const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
     const f16* qp = q + ((int64_t)b * num_heads + g * group + (n < group ? n : 0)) * kPaD + 8 * kg;
+    if constexpr (QLDS) {  // every wave uses the same fragments: wave 0 fetches them
+      if (wave == 0) {
 #pragma unroll
-    for (int s = 0; s < NS; ++s) qreg[s] = n < group ? ld128(qp + 32 * s) : zero8;
+        for (int s = 0; s < NS; ++s)
+          *reinterpret_cast<f16x8*>(sm_q + (s * kWave + lane) * 8) = n < group ? ld128(qp + 32 * s) : zero8;
+      }
+      __syncthreads();
+    } else {
+#pragma unroll
+      for (int s = 0; s < NS; ++s) qreg[s] = n < group ? ld128(qp + 32 * s) : zero8;
+    }
   }
   // Selector operands of the transposing product: sel[u][k][n] = (k == n + 16u), k = 8kg + e.
   f16x8 sel[2];
@@ -266,22 +294,16 @@ __device__ __forceinline__ void pa_process_chunk(
     return page * page_elems + head_off + (int64_t)(tok - (tok / block_size) * block_size) * 16;
   };
 
-  PaRegs<NS> kreg, vreg;
-  int step = wave;
-  if (step < nsteps) {
-    const int64_t off0 = page_offset(step, 0), off1 = page_offset(step, 1);
-    pa_issue_loads(key_cache, off0, off1, lane_off, s_stride, kreg);
-    pa_issue_loads(value_cache, off0, off1, lane_off, s_stride, vreg);
-  }
-  while (step < nsteps) {
-    const int next = step + kPaWaves;
+  // One step of this wave on the register set (kreg, vreg); the set is refilled for the step `stride`
+  // steps further on: K as soon as the scores are out, V as soon as P.V is done.
+  auto do_step = [&](PaRegs<NS>& kreg, PaRegs<NS>& vreg, int step, int stride) {
+    const int next = step + stride;
     const bool has_next = next < nsteps;
     const int64_t next_off0 = has_next ? page_offset(next, 0) : 0;
     const int64_t next_off1 = has_next ? page_offset(next, 1) : 0;
     const int step_token0 = chunk_start + step * kPaStep;
     float sc[8];
-    pa_scores(kreg, qreg, scale_log2, sc);
-    // K registers are free again: the next step's K is in flight during softmax and P.V.
+    pa_scores<NS, QLDS>(kreg, qreg, q_lds, scale_log2, sc);
     if (has_next) pa_issue_loads(key_cache, next_off0, next_off1, lane_off, s_stride, kreg);
     if (step_token0 + kPaStep > context_len) {  // wave uniform: last, partial step of the sequence
       // Cache contents past the end of the sequence are arbitrary (possibly NaN): drop their
@@ -301,8 +323,19 @@ __device__ __forceinline__ void pa_process_chunk(
     const f16x8 pt = pa_softmax(sc, st);
     pa_accumulate(vreg, sel, pt, st);
     if (has_next) pa_issue_loads(value_cache, next_off0, next_off1, lane_off, s_stride, vreg);
-    step = next;
-  }
+  };
+  auto first_loads = [&](PaRegs<NS>& kreg, PaRegs<NS>& vreg, int step) {
+    if (step < nsteps) {
+      const int64_t off0 = page_offset(step, 0), off1 = page_offset(step, 1);
+      pa_issue_loads(key_cache, off0, off1, lane_off, s_stride, kreg);
+      pa_issue_loads(value_cache, off0, off1, lane_off, s_stride, vreg);
+    }
+  };
+  // (A second register set, with the step after next in flight as well, was tried up to head_dim
+  // 128: no gain where it fits, and scratch use in the balanced kernel.)
+  PaRegs<NS> kreg, vreg;
+  first_loads(kreg, vreg, wave);
+  for (int step = wave; step < nsteps; step += kPaWaves) do_step(kreg, vreg, step, kPaWaves);
 
   // The four lanes of a head hold disjoint shares of the sum.
   float l_head = st.l;
