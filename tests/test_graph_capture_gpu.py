@@ -98,6 +98,48 @@ def test_decode_step_and_expert_mlp_in_one_graph(ops, dev):
     torch.testing.assert_close(want[4].cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("B,maxp", [(100, 40), (100, 8), (12, 40)])
+def test_paged_attention_launch_forms_in_a_graph(ops, dev, B, maxp):
+    """The partition of the work is computed on the device at every replay, not at capture: batches of 100
+    sequences with a block table of 5120 tokens (plan kernel + balanced shares + merge) or of 1024 tokens
+    (ranking kernel + whole sequences) and a small batch (in-wave partition), replayed with other context
+    lengths and block tables and compared with the oracle each time."""
+    Hq, Hkv, D, P = 8, 2, 128, 128
+    NB = B * maxp + 4
+    g = torch.Generator().manual_seed(B + maxp)
+    kc_h = R.nz_pack(torch.randn(NB, P, Hkv, D, generator=g).half())
+    vc_h = R.nz_pack(torch.randn(NB, P, Hkv, D, generator=g).half())
+    kc, vc = kc_h.to(dev), vc_h.to(dev)
+
+    def new_inputs(seed):
+        gg = torch.Generator().manual_seed(seed)
+        ctx = torch.randint(0, 300, (B,), generator=gg, dtype=torch.int32)
+        ctx[seed % B] = P * maxp                       # one sequence fills its table row
+        ctx[(seed * 7 + 3) % B] = P * maxp // 2 + 1
+        bt = torch.randperm(NB, generator=gg)[:B * maxp].int().reshape(B, maxp)
+        return torch.randn(B, Hq, D, generator=gg).half(), bt, ctx
+
+    q0, bt0, ctx0 = new_inputs(0)
+    q, bt, ctx = q0.to(dev), bt0.to(dev), ctx0.to(dev)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        ops.paged_attention(q, kc, vc, bt, ctx)
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        o = ops.paged_attention(q, kc, vc, bt, ctx)
+    for seed in (1, 2, 3):
+        qh, bth, ctxh = new_inputs(seed)
+        q.copy_(qh.to(dev)); bt.copy_(bth.to(dev)); ctx.copy_(ctxh.to(dev))
+        graph.replay()
+        torch.cuda.synchronize()
+        ref = R.paged_attention_ref(qh, kc_h, vc_h, bth, ctxh)
+        torch.testing.assert_close(o.cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+        assert torch.equal(o, ops.paged_attention(q, kc, vc, bt, ctx)), f"replay {seed} differs from the eager call"
+
+
 def test_two_streams_concurrently(ops, dev):
     """Entry points keep no device-side state between calls, so independent work on two streams may overlap:
     a grouped matmul chain on one stream and decode attention on the other, several rounds, against the same
