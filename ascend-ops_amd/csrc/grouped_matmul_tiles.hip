@@ -713,7 +713,11 @@ static int matmul_splitk_splits(int64_t m, int64_t k, int64_t n, int cus) {
   return (int)((ktiles + per - 1) / per);  // no empty split
 }
 
-constexpr int kSplitMB = 4, kSplitNB = 2, kSplitWN = 2;  // 256 x 128 tiles, four waves
+// Tiles of the split-k path: 128 columns on four waves, and as many rows as the product has, rounded
+// up to 64, 128 or 256: the fp32 partial results are written and read back tile by tile, so a tile
+// taller than m is wasted traffic (at m <= 64 three quarters of it with 256-row tiles).
+constexpr int kSplitNB = 2, kSplitWN = 2;
+static int splitk_row_blocks(int64_t m) { return m <= 64 ? 1 : m <= 128 ? 2 : 4; }
 
 static int device_cus(int* out) {
   static int cus[64] = {0};  // per device; benign race: every writer stores the same value
@@ -731,20 +735,30 @@ static int device_cus(int* out) {
   return AOPS_OK;
 }
 
-size_t gmm_splitk_workspace(int64_t m, int64_t k, int64_t n) {
-  int cus = 0;
-  if (device_cus(&cus) != AOPS_OK) return 0;
-  const int splits = matmul_splitk_splits<kSplitMB, kSplitNB, kSplitWN>(m, k, n, cus);
+template <int MB>
+static size_t splitk_workspace(int64_t m, int64_t k, int64_t n, int cus) {
+  const int splits = matmul_splitk_splits<MB, kSplitNB, kSplitWN>(m, k, n, cus);
   if (splits < 2) return 0;
-  constexpr int BM = 64 * kSplitMB;
+  constexpr int BM = 64 * MB;
   constexpr int BN = 32 * kSplitNB * kSplitWN;
   const int64_t tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN);
   return (size_t)splits * (size_t)tiles * BM * BN * sizeof(float);
 }
 
-int gmm_launch_splitk(const f16* x, const f16* w, f16* y, float* workspace, size_t workspace_bytes,
-                      int64_t m, int k, int n, hipStream_t stream) {
-  constexpr int MB = kSplitMB, NB = kSplitNB, WN = kSplitWN;
+size_t gmm_splitk_workspace(int64_t m, int64_t k, int64_t n) {
+  int cus = 0;
+  if (device_cus(&cus) != AOPS_OK) return 0;
+  switch (splitk_row_blocks(m)) {
+    case 1: return splitk_workspace<1>(m, k, n, cus);
+    case 2: return splitk_workspace<2>(m, k, n, cus);
+    default: return splitk_workspace<4>(m, k, n, cus);
+  }
+}
+
+template <int MB>
+static int launch_splitk(const f16* x, const f16* w, f16* y, float* workspace, size_t workspace_bytes,
+                         int64_t m, int k, int n, hipStream_t stream) {
+  constexpr int NB = kSplitNB, WN = kSplitWN;
   constexpr int BM = 64 * MB;
   constexpr int BN = 32 * NB * WN;
   int cus = 0;
@@ -773,6 +787,15 @@ int gmm_launch_splitk(const f16* x, const f16* w, f16* y, float* workspace, size
   const int64_t units = tiles * (2 * WN) * MB;  // one wave each
   reduce<<<(unsigned)((units + 3) / 4), 4 * kWave, 0, stream>>>(workspace, y, m, n, splits);
   return record_launch_status(hipGetLastError());
+}
+
+int gmm_launch_splitk(const f16* x, const f16* w, f16* y, float* workspace, size_t workspace_bytes,
+                      int64_t m, int k, int n, hipStream_t stream) {
+  switch (splitk_row_blocks(m)) {
+    case 1: return launch_splitk<1>(x, w, y, workspace, workspace_bytes, m, k, n, stream);
+    case 2: return launch_splitk<2>(x, w, y, workspace, workspace_bytes, m, k, n, stream);
+    default: return launch_splitk<4>(x, w, y, workspace, workspace_bytes, m, k, n, stream);
+  }
 }
 
 template <int MB, int NB, int D, bool SWIGLU = false, bool GATHER = false>

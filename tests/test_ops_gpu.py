@@ -379,7 +379,7 @@ def test_matmul_nt(ops, dev, m, k, n):
 
 
 SPLIT_K_SHAPES = [(256, 14336, 4096), (16, 8192, 1024), (300, 4096, 256), (1, 2048, 64), (257, 64 * 37, 192),
-                  (64, 1024, 2048), (512, 16384, 128)]
+                  (64, 1024, 2048), (100, 2048, 1024), (512, 16384, 128)]
 
 
 @pytest.mark.parametrize("m,k,n", SPLIT_K_SHAPES)
