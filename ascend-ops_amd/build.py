@@ -32,6 +32,7 @@ SOURCES = [
     "grouped_matmul.hip",
     "grouped_matmul_tiles.hip",
     "grouped_matmul_persistent.hip",
+    "matmul_fewrows.hip",
 ]
 
 # -packed-fp32-ops: keep the compiler from forming packed-fp32 VALU instructions.

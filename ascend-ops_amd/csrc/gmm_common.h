@@ -313,6 +313,10 @@ int gmm_launch_tiles_fused(bool small, const f16* x, const f16* w, const int64_t
 // leave most CUs without work.  gmm_splitk_workspace returns the bytes of fp32 scratch the call
 // needs on the current device, 0 when splitting does not pay for the shape.
 size_t gmm_splitk_workspace(int64_t m, int64_t k, int64_t n);
+// Dense products with at most 16 rows of x (matmul_fewrows.hip): one launch, no workspace.
+bool matmul_fewrows_takes(int64_t m, int64_t k, int64_t n);
+int matmul_fewrows_launch(const f16* x, const f16* w, const int64_t* group_list, f16* y, int64_t m, int k,
+                          int n, hipStream_t stream);
 int gmm_launch_splitk(const f16* x, const f16* w, f16* y, float* workspace, size_t workspace_bytes,
                       int64_t m, int k, int n, hipStream_t stream);
 

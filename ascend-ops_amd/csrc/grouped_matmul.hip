@@ -44,6 +44,9 @@ static int aops_grouped_matmul_impl(const void* x, const void* w, const int64_t*
   // rows cover a typical expert of a large routed batch in one tile, and the persistent kernel
   // (320 x 256) wins as soon as there are enough items for one per CU.
   int variant = forced;
+  // a single group of at most 16 rows (the dense projection of a small decode batch): the weight-streaming kernel
+  if ((variant < 1 || variant > 9) && num_experts == 1 && matmul_fewrows_takes(rows, k, n))
+    return matmul_fewrows_launch(xp, wp, group_list, yp, rows, (int)k, (int)n, s);
   if (variant < 1 || variant > 9) {
     const int64_t groups = num_experts < rows ? num_experts : rows;  // experts that can hold a row
     const int64_t avg = (rows + groups - 1) / groups;
@@ -129,6 +132,7 @@ static bool matmul_nt_args_valid(int64_t m, int64_t k, int64_t n) {
 extern "C" size_t aops_matmul_nt_workspace(int64_t m, int64_t k, int64_t n) {
   if (!matmul_nt_args_valid(m, k, n) || m == 0) return 0;
   if (getenv("AOPS_GMM_VARIANT")) return 0;  // a forced kernel choice also switches the k split off
+  if (aops::matmul_fewrows_takes(m, k, n)) return 0;  // one launch, no partial results
   return aops::gmm_splitk_workspace(m, k, n);
 }
 

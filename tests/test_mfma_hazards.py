@@ -8,7 +8,7 @@ import os
 import mfma_hazard_scan as scanner
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-MFMA_SOURCES = ["paged_attention.hip", "grouped_matmul_tiles.hip", "grouped_matmul_persistent.hip"]
+MFMA_SOURCES = ["paged_attention.hip", "grouped_matmul_tiles.hip", "grouped_matmul_persistent.hip", "matmul_fewrows.hip"]
 
 # What the compiler emitted for the paged-attention score product before its accumulators were pinned: the
 # branch is taken when a wave has no further step, and a7 is then read two wait states after its MFMA.

@@ -414,6 +414,42 @@ def test_matmul_nt_split_k(ops, dev, m, k, n):
     assert code == -2 and not out.any()
 
 
+FEW_ROWS_SHAPES = [(1, 4096, 4096), (16, 512, 2048), (7, 576, 2048), (16, 14336, 4096), (9, 4096, 16384),
+                   (5, 2112, 2112)]
+
+
+@pytest.mark.parametrize("m,k,n", FEW_ROWS_SHAPES)
+def test_matmul_nt_few_rows(ops, dev, m, k, n, monkeypatch):
+    """At most 16 rows (the projections of a small decode batch): one workgroup per 16 rows of W, every wave
+    copies its own pieces of W and x into LDS and waits for them alone, no workspace.  Against the fp32 product,
+    against the tile kernels, bit-identical from call to call; through the grouped entry the rows past
+    group_list[0] stay untouched.  k with a short last piece, n that is not a multiple of the XCD run."""
+    import ascend910a_extras.ascend910a_extras_C as C
+
+    g = _gen(m + k + n)
+    x = torch.randn(m, k, generator=g).half()
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).half()
+    xd, wd = x.to(dev), w.to(dev)
+    assert C._lib.aops_matmul_nt_workspace(m, k, n) == 0
+    y = ops.matmul(xd, wd)
+    ref = x.float() @ w.float().T
+    torch.testing.assert_close(y.cpu().float(), ref, **GMM_TOL)
+    assert torch.equal(ops.matmul(xd, wd), y)
+    monkeypatch.setenv("AOPS_GMM_VARIANT", "5")          # the 64 x 64 tile kernel on the same product
+    tiles = ops.matmul(xd, wd)
+    monkeypatch.delenv("AOPS_GMM_VARIANT")
+    torch.testing.assert_close(y.float(), tiles.float(), rtol=2e-3, atol=2e-3)
+    # one group that ends before the last row: later rows are not written
+    part = max(m - 3, 0)
+    gl = torch.tensor([part], dtype=torch.int64, device=dev)
+    out = torch.full((m, n), 7.0, dtype=H, device=dev)
+    code = C._lib.aops_grouped_matmul_f16(xd.data_ptr(), wd.data_ptr(), gl.data_ptr(), out.data_ptr(), m, k, 1, n,
+                                          C._stream(dev))
+    torch.cuda.synchronize()
+    assert code == 0
+    assert torch.equal(out[:part], y[:part]) and bool((out[part:] == 7.0).all())
+
+
 def test_matmul_nt_ws_without_split(ops, dev):
     """Shapes with enough output tiles need no workspace; the workspace entry point then equals the plain one."""
     import ascend910a_extras.ascend910a_extras_C as C
