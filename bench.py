@@ -559,6 +559,14 @@ def bench_mlp(L, ops, R, dev, cpu):
     out.append(e2)
     if cpu:
         torch.testing.assert_close(y_dev.cpu().float(), R.mlp_ref(x, gu, dn).float(), rtol=2e-2, atol=2e-2)
+    # the same hidden size at a decode batch of 16: a square projection as a pure weight stream (extension)
+    xq = torch.randn(16, hidden).half()
+    wq = (0.02 * torch.randn(hidden, hidden)).half()
+    e3, _ = _gmm_entry(L, ops, R, dev, cpu, "grouped_matmul (E=1)", "3 at decode size: 16 rows, 4096 -> 4096",
+                       xq, wq[None], torch.tensor([16], dtype=torch.int64),
+                       note="weight-streaming kernel for at most 16 rows (one launch, no workspace); weight-stream bound")
+    e3["bound"] = "hbm"
+    out.append(e3)
     return out
 
 
