@@ -415,7 +415,7 @@ def test_matmul_nt_split_k(ops, dev, m, k, n):
 
 
 FEW_ROWS_SHAPES = [(1, 4096, 4096), (16, 512, 2048), (7, 576, 2048), (16, 14336, 4096), (9, 4096, 16384),
-                   (5, 2112, 2112)]
+                   (5, 2112, 2112), (4, 14336, 4096), (3, 2112, 2112), (2, 512, 2048), (4, 6208, 2048)]
 
 
 @pytest.mark.parametrize("m,k,n", FEW_ROWS_SHAPES)
