@@ -1,5 +1,7 @@
 // Entry points of libaops that are not operators: version, error text, device summary.
 #include <stdio.h>
+
+#include <atomic>
 #include <string.h>
 
 #include "aops_common.h"
@@ -14,9 +16,30 @@ int record_launch_status(hipError_t e) {
   return AOPS_ERR_LAUNCH;
 }
 
+int device_cu_count() {
+  constexpr int kMaxDevices = 64;
+  constexpr int kDefault = 256;
+  static std::atomic<int> cus[kMaxDevices];  // 0 = not asked yet; every writer stores the same value
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();  // no device: not an error of the caller's launch
+    return kDefault;
+  }
+  if (dev < 0 || dev >= kMaxDevices) return kDefault;
+  int v = cus[dev].load(std::memory_order_relaxed);
+  if (v == 0) {
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) {
+      (void)hipGetLastError();
+      v = kDefault;
+    }
+    cus[dev].store(v, std::memory_order_relaxed);
+  }
+  return v;
+}
+
 }  // namespace aops
 
-extern "C" int aops_version(void) { return 100; }
+extern "C" int aops_version(void) { return 200; }
 
 extern "C" const char* aops_strerror(int code) {
   switch (code) {
@@ -34,6 +57,17 @@ extern "C" const char* aops_strerror(int code) {
 }
 
 extern "C" int aops_last_hip_error(void) { return aops::g_last_hip_error; }
+
+namespace aops {
+__global__ void empty_kernel() {}
+}  // namespace aops
+
+extern "C" int aops_empty_launch(int64_t workgroups, int threads, void* stream) {
+  if (workgroups <= 0 || workgroups > 0x7fffffff || threads <= 0 || threads > 1024)
+    return AOPS_ERR_INVALID_ARGUMENT;
+  aops::empty_kernel<<<(unsigned)workgroups, (unsigned)threads, 0, static_cast<hipStream_t>(stream)>>>();
+  return aops::record_launch_status(hipGetLastError());
+}
 
 extern "C" int aops_device_info(int device, char* buf, size_t buf_len) {
   if (!buf || buf_len == 0) return AOPS_ERR_INVALID_ARGUMENT;

@@ -86,4 +86,9 @@ __device__ __forceinline__ uint32_t xcd_run_index(uint32_t wg, uint32_t num_wgs)
 // Launch-status bookkeeping shared by the host launchers.
 int record_launch_status(hipError_t e);
 
+// Compute units of the current device (queried once per device; 256, an MI355X, when there is no
+// device to ask).  The one source of the CU count for every launcher that sizes a grid or a
+// partition by it.
+int device_cu_count();
+
 }  // namespace aops

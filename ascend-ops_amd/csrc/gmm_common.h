@@ -317,7 +317,8 @@ size_t gmm_splitk_workspace(int64_t m, int64_t k, int64_t n);
 bool matmul_fewrows_takes(int64_t m, int64_t k, int64_t n);
 int matmul_fewrows_launch(const f16* x, const f16* w, const int64_t* group_list, f16* y, int64_t m, int k,
                           int n, hipStream_t stream);
-int gmm_launch_splitk(const f16* x, const f16* w, f16* y, float* workspace, size_t workspace_bytes,
-                      int64_t m, int k, int n, hipStream_t stream);
+// group_list != nullptr: the single group ends at group_list[0]; rows behind it are not written.
+int gmm_launch_splitk(const f16* x, const f16* w, const int64_t* group_list, f16* y, float* workspace,
+                      size_t workspace_bytes, int64_t m, int k, int n, hipStream_t stream);
 
 }  // namespace aops

@@ -16,13 +16,12 @@
 // Semantics: reference csrc/opdev/op_kernel/grouped_mat_mul_ex.cpp:27-44 (start/end from the
 // cumulative int64 group_list, empty groups skipped), matmul_core.h:42-68 (NT product, fp32
 // accumulate, fp16 result), benchmark/test_grouped_matmul.py:6-23.
-#include <stdlib.h>
-
 #include "gmm_common.h"
 
+// forced: 1..9 = that kernel / tile shape whatever the problem size (the override entry point), 0 = choose.
 static int aops_grouped_matmul_impl(const void* x, const void* w, const int64_t* group_list, void* y,
                                     int64_t rows, int64_t k, int64_t num_experts, int64_t n,
-                                    void* stream) {
+                                    void* stream, int forced = 0) {
   using namespace aops;
   if (rows < 0 || k <= 0 || n <= 0 || num_experts < 0 || k % 64 != 0 || n % 64 != 0)
     return AOPS_ERR_INVALID_ARGUMENT;
@@ -35,8 +34,6 @@ static int aops_grouped_matmul_impl(const void* x, const void* w, const int64_t*
   const f16* xp = static_cast<const f16*>(x);
   const f16* wp = static_cast<const f16*>(w);
   f16* yp = static_cast<f16*>(y);
-  const char* forced_env = getenv("AOPS_GMM_VARIANT");  // tuning aid: 1..9 force one kernel / tile shape
-  const int forced = forced_env ? atoi(forced_env) : 0;
   // Tile choice from what the host knows (group_list stays on the device, so the rows are taken
   // to be spread evenly over the experts).  With few rows per expert the weights are streamed for
   // little arithmetic and every tile row beyond the group is wasted copy and MFMA work: 128- or
@@ -52,7 +49,7 @@ static int aops_grouped_matmul_impl(const void* x, const void* w, const int64_t*
     const int64_t avg = (rows + groups - 1) / groups;
     auto m_tiles = [&](int64_t bm) { return (avg + bm - 1) / bm; };
     auto items = [&](int64_t bm, int64_t bn) { return groups * m_tiles(bm) * ((n + bn - 1) / bn); };
-    constexpr int64_t kEnough = 190;  // of 256 CUs
+    const int64_t kEnough = (int64_t)device_cu_count() * 3 / 4;  // items that still keep most CUs busy
     if (avg < 96) {
       variant = (avg >= 24 && items(128, 128) >= kEnough) ? 4 : 5;
     } else if (items(320, 256) >= kEnough) {
@@ -81,6 +78,14 @@ extern "C" int aops_grouped_matmul_f16(const void* x, const void* w, const int64
                                        int64_t n, void* stream) {
   if (rows > 0 && num_experts > 0 && !group_list) return AOPS_ERR_INVALID_ARGUMENT;
   return aops_grouped_matmul_impl(x, w, group_list, y, rows, k, num_experts, n, stream);
+}
+
+extern "C" int aops_grouped_matmul_variant_f16(int variant, const void* x, const void* w,
+                                               const int64_t* group_list, void* y, int64_t rows,
+                                               int64_t k, int64_t num_experts, int64_t n,
+                                               void* stream) {
+  if (variant < 1 || variant > 9) return AOPS_ERR_INVALID_ARGUMENT;
+  return aops_grouped_matmul_impl(x, w, group_list, y, rows, k, num_experts, n, stream, variant);
 }
 
 // Kernel choice of the fused entry points: 0 = persistent 320 x 256 kernel, 1 = 128 x 128 tiles,
@@ -131,7 +136,6 @@ static bool matmul_nt_args_valid(int64_t m, int64_t k, int64_t n) {
 
 extern "C" size_t aops_matmul_nt_workspace(int64_t m, int64_t k, int64_t n) {
   if (!matmul_nt_args_valid(m, k, n) || m == 0) return 0;
-  if (getenv("AOPS_GMM_VARIANT")) return 0;  // a forced kernel choice also switches the k split off
   if (aops::matmul_fewrows_takes(m, k, n)) return 0;  // one launch, no partial results
   return aops::gmm_splitk_workspace(m, k, n);
 }
@@ -144,9 +148,25 @@ extern "C" int aops_matmul_nt_ws_f16(const void* x, const void* w, void* y, void
   if (!x || !w || !y) return AOPS_ERR_INVALID_ARGUMENT;
   if (aops_matmul_nt_workspace(m, k, n) == 0)
     return aops_grouped_matmul_impl(x, w, nullptr, y, m, k, 1, n, stream);
-  return aops::gmm_launch_splitk(static_cast<const aops::f16*>(x), static_cast<const aops::f16*>(w),
+  return aops::gmm_launch_splitk(static_cast<const aops::f16*>(x), static_cast<const aops::f16*>(w), nullptr,
                                  static_cast<aops::f16*>(y), static_cast<float*>(workspace),
                                  workspace_bytes, m, (int)k, (int)n, static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t aops_grouped_matmul_workspace(int64_t rows, int64_t k, int64_t num_experts, int64_t n) {
+  // only a single group of few rows with a long k is split over k; every other shape needs no scratch
+  return num_experts == 1 ? aops_matmul_nt_workspace(rows, k, n) : 0;
+}
+
+extern "C" int aops_grouped_matmul_ws_f16(const void* x, const void* w, const int64_t* group_list, void* y,
+                                          void* workspace, size_t workspace_bytes, int64_t rows, int64_t k,
+                                          int64_t num_experts, int64_t n, void* stream) {
+  if (aops_grouped_matmul_workspace(rows, k, num_experts, n) == 0)
+    return aops_grouped_matmul_f16(x, w, group_list, y, rows, k, num_experts, n, stream);
+  if (!x || !w || !y || !group_list) return AOPS_ERR_INVALID_ARGUMENT;
+  return aops::gmm_launch_splitk(static_cast<const aops::f16*>(x), static_cast<const aops::f16*>(w), group_list,
+                                 static_cast<aops::f16*>(y), static_cast<float*>(workspace),
+                                 workspace_bytes, rows, (int)k, (int)n, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int aops_grouped_matmul_swiglu_gather_f16(const void* x, const int32_t* row_idx,

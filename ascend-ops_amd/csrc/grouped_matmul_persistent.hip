@@ -358,28 +358,18 @@ static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* grou
   constexpr int kWaves = 2 * WN;
   constexpr int kLds = 2 * (BM + BN) * kBK * (int)sizeof(f16) + kWaves * kWave * 8 * (int)sizeof(int);
   static_assert(kLds <= 160 * 1024, "LDS budget");
-  static int cus[64] = {0};  // per device; benign race: every writer stores the same value
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return record_launch_status(e);
-  if (dev < 0 || dev >= 64) return AOPS_ERR_INVALID_ARGUMENT;
-  if (cus[dev] == 0) {
-    int v = 0;
-    e = hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e != hipSuccess) return record_launch_status(e);
-    cus[dev] = v > 0 ? v : 8;
-  }
+  const int cus = device_cu_count();
   constexpr int BNO = SWIGLU ? BN / 2 : BN;
   const int64_t n_out = SWIGLU ? n / 2 : n;
   const int64_t n_tiles = (n_out + BNO - 1) / BNO;
   const int64_t max_work = ((rows + BM - 1) / BM + num_experts) * n_tiles;
-  int64_t grid = cus[dev] < max_work ? cus[dev] : max_work;
+  int64_t grid = cus < max_work ? cus : max_work;
   grid = grid / kXcds * kXcds;
   if (grid < kXcds) grid = kXcds;
   auto kernel = grouped_matmul_persistent_kernel<MB, NB, WN, SWIGLU, GATHER>;
   static bool attr_set = false;  // benign race: the call is idempotent
   if (!attr_set) {
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
     if (e != hipSuccess) return record_launch_status(e);
     attr_set = true;
@@ -413,7 +403,7 @@ int gmm_launch_persistent(bool swiglu, const f16* x, const f16* w, const int64_t
                           int64_t rows, int k, int num_experts, int n, hipStream_t stream,
                           const int32_t* row_idx, int idx_div, int64_t x_rows) {
   const int64_t n_out_tiles = swiglu ? (n / 2 + 127) / 128 : (n + 255) / 256;
-  const bool small = gmm_prefer_256_rows(rows, num_experts, n_out_tiles, 256);
+  const bool small = gmm_prefer_256_rows(rows, num_experts, n_out_tiles, device_cu_count());
   if (row_idx) {  // only the fused gate_up form gathers
     if (small)
       return gmm_persistent_launch<4, 2, 4, true, true>(x, w, group_list, y, rows, k, num_experts, n, stream,

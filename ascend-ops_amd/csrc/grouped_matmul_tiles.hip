@@ -623,7 +623,8 @@ static int gmm_dma_launch(const f16* x, const f16* w, const int64_t* group_list,
 // No LDS, no barrier; the loads of all splits are independent.
 template <int MB, int NB, int WN>
 __global__ __launch_bounds__(4 * kWave) void matmul_splitk_reduce(
-    const float* __restrict__ partial, f16* __restrict__ y, int64_t rows, int n, int splits) {
+    const float* __restrict__ partial, f16* __restrict__ y, int64_t rows, int n, int splits,
+    const int64_t* __restrict__ group_list) {
   constexpr int kWaves = 2 * WN;
   constexpr int BM = 64 * MB;
   constexpr int BN = 32 * NB * WN;
@@ -667,7 +668,9 @@ __global__ __launch_bounds__(4 * kWave) void matmul_splitk_reduce(
   // acc[j][g][e]: row 32*(wm + 2i) + fm, column wn*32*NB + 32j + 8g + 4fq + e of the tile
   const int m = 32 * (wm + 2 * i) + fm;
   const int col_w = n_tile * BN + wn * 32 * NB;
-  const bool row_ok = m < tile_rows;
+  // a single group that ends before the last row: the rows behind it are not written
+  const int64_t row_limit = group_list ? min(max(group_list[0], (int64_t)0), rows) : rows;
+  const bool row_ok = m < tile_rows && row_begin + m < row_limit;
   f16* yrow = y + (int64_t)(row_begin + m) * n + col_w + 8 * fq;
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
@@ -719,22 +722,6 @@ static int matmul_splitk_splits(int64_t m, int64_t k, int64_t n, int cus) {
 constexpr int kSplitNB = 2, kSplitWN = 2;
 static int splitk_row_blocks(int64_t m) { return m <= 64 ? 1 : m <= 128 ? 2 : 4; }
 
-static int device_cus(int* out) {
-  static int cus[64] = {0};  // per device; benign race: every writer stores the same value
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return record_launch_status(e);
-  if (dev < 0 || dev >= 64) return AOPS_ERR_INVALID_ARGUMENT;
-  if (cus[dev] == 0) {
-    int v = 0;
-    e = hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e != hipSuccess) return record_launch_status(e);
-    cus[dev] = v > 0 ? v : 8;
-  }
-  *out = cus[dev];
-  return AOPS_OK;
-}
-
 template <int MB>
 static size_t splitk_workspace(int64_t m, int64_t k, int64_t n, int cus) {
   const int splits = matmul_splitk_splits<MB, kSplitNB, kSplitWN>(m, k, n, cus);
@@ -746,8 +733,7 @@ static size_t splitk_workspace(int64_t m, int64_t k, int64_t n, int cus) {
 }
 
 size_t gmm_splitk_workspace(int64_t m, int64_t k, int64_t n) {
-  int cus = 0;
-  if (device_cus(&cus) != AOPS_OK) return 0;
+  const int cus = device_cu_count();
   switch (splitk_row_blocks(m)) {
     case 1: return splitk_workspace<1>(m, k, n, cus);
     case 2: return splitk_workspace<2>(m, k, n, cus);
@@ -756,15 +742,12 @@ size_t gmm_splitk_workspace(int64_t m, int64_t k, int64_t n) {
 }
 
 template <int MB>
-static int launch_splitk(const f16* x, const f16* w, f16* y, float* workspace, size_t workspace_bytes,
-                         int64_t m, int k, int n, hipStream_t stream) {
+static int launch_splitk(const f16* x, const f16* w, const int64_t* group_list, f16* y, float* workspace,
+                         size_t workspace_bytes, int64_t m, int k, int n, hipStream_t stream) {
   constexpr int NB = kSplitNB, WN = kSplitWN;
   constexpr int BM = 64 * MB;
   constexpr int BN = 32 * NB * WN;
-  int cus = 0;
-  const int rc = device_cus(&cus);
-  if (rc != AOPS_OK) return rc;
-  const int splits = matmul_splitk_splits<MB, NB, WN>(m, k, n, cus);
+  const int splits = matmul_splitk_splits<MB, NB, WN>(m, k, n, device_cu_count());
   const int64_t tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN);
   if (splits < 2) return AOPS_ERR_INVALID_ARGUMENT;
   if (!workspace || workspace_bytes < (size_t)splits * (size_t)tiles * BM * BN * sizeof(float))
@@ -785,16 +768,16 @@ static int launch_splitk(const f16* x, const f16* w, f16* y, float* workspace, s
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return record_launch_status(e);
   const int64_t units = tiles * (2 * WN) * MB;  // one wave each
-  reduce<<<(unsigned)((units + 3) / 4), 4 * kWave, 0, stream>>>(workspace, y, m, n, splits);
+  reduce<<<(unsigned)((units + 3) / 4), 4 * kWave, 0, stream>>>(workspace, y, m, n, splits, group_list);
   return record_launch_status(hipGetLastError());
 }
 
-int gmm_launch_splitk(const f16* x, const f16* w, f16* y, float* workspace, size_t workspace_bytes,
-                      int64_t m, int k, int n, hipStream_t stream) {
+int gmm_launch_splitk(const f16* x, const f16* w, const int64_t* group_list, f16* y, float* workspace,
+                      size_t workspace_bytes, int64_t m, int k, int n, hipStream_t stream) {
   switch (splitk_row_blocks(m)) {
-    case 1: return launch_splitk<1>(x, w, y, workspace, workspace_bytes, m, k, n, stream);
-    case 2: return launch_splitk<2>(x, w, y, workspace, workspace_bytes, m, k, n, stream);
-    default: return launch_splitk<4>(x, w, y, workspace, workspace_bytes, m, k, n, stream);
+    case 1: return launch_splitk<1>(x, w, group_list, y, workspace, workspace_bytes, m, k, n, stream);
+    case 2: return launch_splitk<2>(x, w, group_list, y, workspace, workspace_bytes, m, k, n, stream);
+    default: return launch_splitk<4>(x, w, group_list, y, workspace, workspace_bytes, m, k, n, stream);
   }
 }
 

@@ -30,8 +30,6 @@
 // Semantics: signature, cache indexing, GQA mapping and the fixed 1/sqrt(D) scale follow
 // reference csrc/ffi/ops.cpp:408-482, csrc/opdev/op_host/paged_attention_ex.cpp:18-36 and
 // csrc/opdev/op_kernel/paged_attention_ex.cpp:90-99 (whose compute body is unfinished).
-#include <stdlib.h>
-
 #include "aops_common.h"
 
 namespace aops {
@@ -48,6 +46,7 @@ struct PaChunking {
 };
 
 constexpr int kPaUnit = kPaWaves * kPaStep;  // 256 tokens: one step of every wave
+constexpr int kPaMaxGroup = 16;              // query heads per kv head the matrix-core kernel serves
 
 // Batches of up to kPaPlanMax sequences can use the balanced partition; above 64 sequences it is
 // computed by a one-workgroup kernel into kPaPlanInts(bs) ints behind the partial results.
@@ -58,23 +57,18 @@ static size_t pa_tail_ints(int64_t bs) { return bs <= 64 ? (size_t)bs : (size_t)
 
 static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_size,
                               int64_t max_blocks_per_seq) {
+  const int64_t cus = device_cu_count();
   const int64_t max_len = block_size * max_blocks_per_seq;
   // As few chunks per sequence as still give every CU two workgroups: each chunk costs a
   // partial result and a workgroup prologue, and long chunks keep the load stream steady.
   constexpr int kUnit = kPaWaves * kPaStep;
-  constexpr int64_t kWantedWorkgroups = 512;
-  int64_t splits = (kWantedWorkgroups + bs * num_kv_heads - 1) / (bs * num_kv_heads > 0 ? bs * num_kv_heads : 1);
+  const int64_t wanted_workgroups = 2 * cus;
+  int64_t splits = (wanted_workgroups + bs * num_kv_heads - 1) / (bs * num_kv_heads > 0 ? bs * num_kv_heads : 1);
   const int64_t max_units = (max_len + kUnit - 1) / kUnit;
   if (splits > max_units) splits = max_units;
   if (splits < 1) splits = 1;
   int chunk = (int)(((max_units + splits - 1) / splits) * kUnit);
   if (chunk < kUnit) chunk = kUnit;
-  static const int forced = [] {
-    const char* e = getenv("AOPS_PA_CHUNK");  // tuning aid; a multiple of 256 tokens, ignored otherwise
-    const int v = e ? atoi(e) : 0;
-    return (v >= kPaWaves * kPaStep && v % (kPaWaves * kPaStep) == 0) ? v : 0;
-  }();
-  if (forced) chunk = forced;
   if ((max_len + chunk - 1) / chunk > kPaMaxChunks)  // the merge kernel keeps one weight per chunk in LDS
     chunk = (int)(((max_units + kPaMaxChunks - 1) / kPaMaxChunks) * kUnit);
   PaChunking c;
@@ -85,18 +79,11 @@ static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_si
   // Small batches: fixed chunks of a few long sequences either leave CUs idle or, cut finer, pay
   // the per-workgroup start-up many times over.  With fewer than two (sequence, kv head) pairs per
   // CU the token stream is cut into one equal share per CU instead.
-  static const int balanced_env = [] {
-    const char* e = getenv("AOPS_PA_BALANCED");  // tuning aid: 0 = off, n = n workgroups in total
-    return e ? atoi(e) : -1;
-  }();
-  constexpr int64_t kCus = 256;
   // ... and whenever the block table allows contexts beyond 4096 tokens: whole sequences per workgroup
   // would let one long sequence among short ones occupy eight CUs for the whole launch.
   constexpr int64_t kSkewFreeLen = 4096;
-  if (!forced && balanced_env != 0 && bs <= kPaPlanMax && max_units >= 2 &&
-      (bs * num_kv_heads < 2 * kCus || max_len > kSkewFreeLen || balanced_env > 0)) {
-    const int64_t total = balanced_env > 0 ? balanced_env : kCus;
-    int64_t wgs = (total + num_kv_heads - 1) / num_kv_heads;
+  if (bs <= kPaPlanMax && max_units >= 2 && (bs * num_kv_heads < 2 * cus || max_len > kSkewFreeLen)) {
+    int64_t wgs = (cus + num_kv_heads - 1) / num_kv_heads;
     if (wgs > kPaMaxShares) wgs = kPaMaxShares;
     if (wgs > bs * max_units) wgs = bs * max_units;  // never more shares than units
     c.balanced_wgs = (int)wgs;
@@ -828,8 +815,10 @@ static bool pa_args_valid(int64_t bs, int64_t num_heads, int64_t num_kv_heads, i
 static bool pa_fast_shape(int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
                           int64_t block_size) {
   if ((head_dim != 64 && head_dim != 128 && head_dim != 256) || block_size % 16 != 0) return false;
-  // the cross-wave merge keeps 8 x group x head_dim floats in LDS: at most 66 KB
-  return (num_heads / num_kv_heads) * head_dim <= 16 * 128;
+  // a lane of the score product holds one of at most 16 query heads of the kv head, and the cross-wave
+  // merge keeps 8 x group x head_dim floats in LDS (at most 66 KB): up to 16 heads, 8 at head_dim 256
+  const int64_t group = num_heads / num_kv_heads;
+  return group <= kPaMaxGroup && group * head_dim <= kPaMaxGroup * 128;
 }
 
 }  // namespace aops
@@ -847,14 +836,15 @@ extern "C" size_t aops_paged_attention_workspace(int64_t bs, int64_t num_heads,
          pa_tail_ints(bs) * sizeof(int32_t);
 }
 
-extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
-                                        const void* value_cache, const int32_t* block_tables,
-                                        const int32_t* context_lens, void* o, void* workspace,
-                                        size_t workspace_bytes, int64_t bs, int64_t num_heads,
-                                        int64_t num_kv_heads, int64_t head_dim,
-                                        int64_t block_size, int64_t max_blocks_per_seq,
-                                        int64_t num_blocks, void* stream) {
-  using namespace aops;
+namespace aops {
+
+// The work of both entry points: argument checks, kernel choice, launches.  `workspace` is device
+// memory of at least aops_paged_attention_workspace(...) bytes (not touched by the generic kernel).
+static int pa_run(const void* q, const void* key_cache, const void* value_cache,
+                  const int32_t* block_tables, const int32_t* context_lens, void* o, void* workspace,
+                  size_t workspace_bytes, int64_t bs, int64_t num_heads, int64_t num_kv_heads,
+                  int64_t head_dim, int64_t block_size, int64_t max_blocks_per_seq,
+                  int64_t num_blocks, void* stream) {
   if (!pa_args_valid(bs, num_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq) ||
       num_blocks < 0 || num_blocks > 0x7fffffff)
     return AOPS_ERR_INVALID_ARGUMENT;
@@ -898,6 +888,7 @@ extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
     AOPS_PA_CASE(D, 16)       \
   }
   const int64_t group = num_heads / num_kv_heads;
+  if (group > kPaMaxGroup) return AOPS_ERR_INVALID_ARGUMENT;  // pa_fast_shape admits no such shape
   const int gmax = group <= 1 ? 1 : group <= 2 ? 2 : group <= 4 ? 4 : group <= 8 ? 8 : 16;
   if (head_dim == 64) {
     AOPS_PA_GROUPS(64)
@@ -909,4 +900,18 @@ extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
 #undef AOPS_PA_GROUPS
 #undef AOPS_PA_CASE
   return record_launch_status(hipGetLastError());
+}
+
+}  // namespace aops
+
+extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
+                                        const void* value_cache, const int32_t* block_tables,
+                                        const int32_t* context_lens, void* o, void* workspace,
+                                        size_t workspace_bytes, int64_t bs, int64_t num_heads,
+                                        int64_t num_kv_heads, int64_t head_dim,
+                                        int64_t block_size, int64_t max_blocks_per_seq,
+                                        int64_t num_blocks, void* stream) {
+  return aops::pa_run(q, key_cache, value_cache, block_tables, context_lens, o, workspace,
+                      workspace_bytes, bs, num_heads, num_kv_heads, head_dim, block_size,
+                      max_blocks_per_seq, num_blocks, stream);
 }

@@ -11,7 +11,9 @@
 //
 // NORM = true puts the per-head RMSNorm of q and k (reference csrc/ffi/graph.cpp:252-253: RMSNorm
 // without residual over head_dim, one weight vector for q and one for k) in front of the rotation:
-// the head_dim/16 threads of a head add up their squares with lane exchanges, the normalised
+// the head_dim/16 threads of a head add up their squares with lane exchanges (when that count is a
+// power of two, so that a head's threads are aligned lanes of one wave; for any other head size
+// every thread adds up its whole head itself from loads its neighbours share), the normalised
 // values are rounded to fp16 as the separate operator's output would be, then rotated.
 #include "aops_common.h"
 
@@ -67,10 +69,20 @@ __global__ __launch_bounds__(256) void rope_cache_kernel(
     const f16x8 w1 = ld128(nw + c * 8);
     const f16x8 w2 = ld128(nw + half + c * 8);
     float ss = 0.f;
+    if ((vec_per_head & (vec_per_head - 1)) == 0 && vec_per_head <= 16) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) ss += (float)x1[j] * (float)x1[j] + (float)x2[j] * (float)x2[j];
-    // the vec_per_head (a power of two) threads of this head are consecutive, aligned lanes
-    for (uint32_t m = 1; m < vec_per_head; m <<= 1) ss += __shfl_xor(ss, (int)m);
+      for (int j = 0; j < 8; ++j) ss += (float)x1[j] * (float)x1[j] + (float)x2[j] * (float)x2[j];
+      // the vec_per_head threads of this head are consecutive, aligned lanes
+      for (uint32_t m = 1; m < vec_per_head; m <<= 1) ss += __shfl_xor(ss, (int)m);
+    } else {
+      // a head's threads may lie in two waves or workgroups: every thread sums the head, all in the
+      // same order, so they agree on the result bit for bit
+      for (uint32_t p = 0; p < head_dim / 8; ++p) {
+        const f16x8 xv = ld128(src + base + p * 8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss += (float)xv[j] * (float)xv[j];
+      }
+    }
     const float inv_rms = 1.0f / __builtin_sqrtf(ss / (float)head_dim + eps);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -108,9 +120,6 @@ static int rope_cache_launch(bool norm, const void* q, const void* k, const void
                              int64_t block_size, void* stream) {
   if (bs < 0 || num_heads < 0 || num_kv_heads <= 0 || head_dim <= 0 || head_dim % 16 != 0 ||
       num_blocks < 0 || block_size <= 0 || block_size > 0x7fffffff)
-    return AOPS_ERR_INVALID_ARGUMENT;
-  // the norm's lane exchange needs head_dim/16 threads per head to be a power of two up to 16
-  if (norm && (head_dim > 256 || ((head_dim / 16) & (head_dim / 16 - 1)) != 0))
     return AOPS_ERR_INVALID_ARGUMENT;
   const int64_t num_slots = num_blocks * block_size;
   if (num_slots > 0x7fffffff) return AOPS_ERR_INVALID_ARGUMENT;  // slots are int32

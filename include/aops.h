@@ -114,7 +114,7 @@ int aops_rope_reshape_and_cache_f16(const void* q, const void* k, const void* v,
  * csrc/ffi/graph.cpp:252-253: RMSNorm over head_dim without residual, weights [head_dim]):
  *   qn = f16( q * rsqrt(mean(q^2 over the head) + epsilon) * q_norm_weight ), likewise kn;
  *   out_q = rope(qn); rotated kn and v go to the caches.
- * head_dim must be 16, 32, 64, 128 or 256.  Equal to the chain of the separate operators up to the
+ * head_dim: any multiple of 16.  Equal to the chain of the separate operators up to the
  * summation order of the mean (within the operators' tolerance, not bit for bit).
  */
 int aops_qknorm_rope_reshape_and_cache_f16(
@@ -138,6 +138,36 @@ int aops_qknorm_rope_reshape_and_cache_f16(
 int aops_grouped_matmul_f16(const void* x, const void* w, const int64_t* group_list, void* y,
                             int64_t rows, int64_t k, int64_t num_experts, int64_t n,
                             void* stream);
+
+/*
+ * Two-phase form of aops_grouped_matmul_f16, the reference's own calling convention
+ * (aclnnGroupedMatMulExGetWorkspaceSize, then aclnnGroupedMatMulEx with the workspace: reference
+ * csrc/ffi/ops.cpp:211-218).  aops_grouped_matmul_workspace returns the bytes of device scratch the
+ * call wants on the current device: non-zero only for one expert with few rows and a long k, which
+ * then runs the k-split kernels of aops_matmul_nt_ws_f16 (rows at or past group_list[0] are not
+ * written, as everywhere); 0 = no scratch, and aops_grouped_matmul_ws_f16 does exactly what
+ * aops_grouped_matmul_f16 does.  A workspace that is wanted but missing or too small returns
+ * AOPS_ERR_WORKSPACE.
+ */
+size_t aops_grouped_matmul_workspace(int64_t rows, int64_t k, int64_t num_experts, int64_t n);
+int aops_grouped_matmul_ws_f16(const void* x, const void* w, const int64_t* group_list, void* y,
+                               void* workspace, size_t workspace_bytes, int64_t rows, int64_t k,
+                               int64_t num_experts, int64_t n, void* stream);
+
+/*
+ * aops_grouped_matmul_f16 with the kernel fixed by the caller instead of chosen from the problem
+ * size: for tests (every kernel over every edge case) and tuning sweeps.  variant 1 = 320 x 256 tiles
+ * with direct HBM -> LDS copies, one workgroup per tile; 2 = 320 x 128, 3 = 256 x 128, 4 = 128 x 128,
+ * 5 = 64 x 64 register-staged tiles; 6 = the persistent 320 x 256 kernel (k % 128 == 0, k >= 256, else
+ * variant 1); 7 = 256 x 128, 8 = 128 x 128 direct copies; 9 = 256 x 128 with three LDS stages.  Any
+ * other value returns AOPS_ERR_INVALID_ARGUMENT.  With num_experts == 1, group_list may be NULL (one
+ * group that holds every row).  Same results as aops_grouped_matmul_f16 within fp16 rounding.
+ * No counterpart in the reference, whose kernel has one tile shape (reference
+ * csrc/opdev/op_kernel/matmul_core.h:8-40).
+ */
+int aops_grouped_matmul_variant_f16(int variant, const void* x, const void* w,
+                                    const int64_t* group_list, void* y, int64_t rows, int64_t k,
+                                    int64_t num_experts, int64_t n, void* stream);
 
 /*
  * Dense NT matmul: y = f16( x (fp32 accumulate) @ w^T ), x: [m, k], w: [n, k], y: [m, n]; the
@@ -255,6 +285,14 @@ int aops_paged_attention_f16(const void* q, const void* key_cache, const void* v
                              int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
                              int64_t block_size, int64_t max_blocks_per_seq, int64_t num_blocks,
                              void* stream);
+
+/*
+ * Measurement aid: launches a kernel that does nothing, `workgroups` workgroups of `threads` threads
+ * (1..1024).  Its duration is the floor that any launch of that geometry pays for dispatch, ramp-up
+ * and drain: what a latency-bound operator (a few MB of traffic) is up against besides HBM.
+ * No counterpart in the reference.
+ */
+int aops_empty_launch(int64_t workgroups, int threads, void* stream);
 
 /*
  * Device summary (CU count, LDS, L2, memory size, clocks) written as text into buf
