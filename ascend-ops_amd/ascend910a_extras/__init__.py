@@ -2,13 +2,27 @@
 
 Same module layout as the reference package (reference
 ``ascend910a_extras/__init__.py:1-27``, which dlopens its operator library at
-import): importing this package loads ``libaops.so`` -- the C-ABI library of
-hand-written HIP kernels -- and fails loudly if it is missing.  There is no
-CPU or eager fallback.
+import and then imports its pybind module): importing this package loads the
+torch extension module ``ascend910a_extras_C`` and, through it, ``libaops.so``
+-- the C-ABI library of hand-written HIP kernels -- and fails loudly if either
+is missing.  There is no CPU or eager fallback.
 """
-from . import ascend910a_extras_C  # noqa: F401  (loads libaops.so)
-from . import ops  # noqa: F401
-from . import fused  # noqa: F401
-from . import moe  # noqa: F401
+import glob as _glob
+import os as _os
 
-__all__ = ["ops", "fused", "moe", "ascend910a_extras_C"]
+import torch  # noqa: F401  (the extension module links against torch's libraries)
+
+_here = _os.path.dirname(_os.path.abspath(__file__))
+LIBRARY_PATH = _os.path.join(_here, "libaops.so")
+if not _os.path.exists(LIBRARY_PATH) or not _glob.glob(_os.path.join(_here, "ascend910a_extras_C.*.so")):
+    raise ImportError(
+        f"{_here} lacks libaops.so or the ascend910a_extras_C extension module: the HIP kernel library has "
+        "not been built (run `python ascend-ops_amd/build.py`). There is no fallback implementation."
+    )
+
+from . import ascend910a_extras_C  # noqa: E402,F401  (loads libaops.so)
+from . import ops  # noqa: E402,F401
+from . import fused  # noqa: E402,F401
+from . import moe  # noqa: E402,F401
+
+__all__ = ["ops", "fused", "moe", "ascend910a_extras_C", "LIBRARY_PATH"]

@@ -1,8 +1,11 @@
-"""Builds libaops.so (the C-ABI library of gfx950 HIP kernels) in-tree with hipcc.
+"""Builds, in-tree, the two native parts of the package:
 
-Usage: ``python build.py [--force]`` or ``from build import build_library``.
-The library is written next to the Python package that loads it
-(``ascend910a_extras/libaops.so``).
+* ``ascend910a_extras/libaops.so``: the C-ABI library of gfx950 HIP kernels (hipcc);
+* ``ascend910a_extras/ascend910a_extras_C<ext suffix>``: the torch extension module that the Python API
+  calls (host C++ only: argument checks, output allocation, current HIP stream, one ``aops_*`` call per
+  operator), compiled with the C++ compiler against the torch headers and linked against ``libaops.so``.
+
+Usage: ``python build.py [--force]`` or ``from build import build_all``.
 """
 from __future__ import annotations
 
@@ -10,6 +13,7 @@ import os
 import shutil
 import subprocess
 import sys
+import sysconfig
 from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
@@ -120,6 +124,57 @@ def emit_assembly(out_dir: Path, sources=None) -> list:
         return list(pool.map(one, names))
 
 
+EXT_NAME = "ascend910a_extras_C"
+EXT_SOURCE = CSRC / "binding" / "ascend910a_extras_C.cpp"
+
+
+def extension_path() -> Path:
+    return OUT_DIR / (EXT_NAME + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_extension(force: bool = True, verbose: bool = False) -> Path:
+    """Compiles the torch extension module (host C++) and links it against libaops.so and torch."""
+    import torch
+    from torch.utils import cpp_extension
+
+    out = extension_path()
+    lib = library_path()
+    if not lib.exists():
+        raise RuntimeError(f"{lib} must be built first")
+    deps = [EXT_SOURCE, INCLUDE / "aops.h"]
+    if not force and out.exists() and out.stat().st_mtime >= max(d.stat().st_mtime for d in deps):
+        return out
+    cxx = shutil.which(os.environ.get("CXX", "g++")) or shutil.which("c++")
+    if not cxx:
+        raise RuntimeError("no C++ compiler found: the torch extension cannot be built")
+    torch_lib = Path(torch.__file__).resolve().parent / "lib"
+    includes = [str(INCLUDE), *cpp_extension.include_paths("cuda"), sysconfig.get_paths()["include"]]
+    tmp = out.with_suffix(".tmp")
+    cmd = [
+        cxx, "-O2", "-fPIC", "-shared", "-std=c++17", "-fvisibility=hidden",
+        "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+        f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+        f"-DTORCH_EXTENSION_NAME={EXT_NAME}",
+        *[f"-I{p}" for p in includes],
+        str(EXT_SOURCE), "-o", str(tmp),
+        f"-L{OUT_DIR}", "-laops",
+        f"-L{torch_lib}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python",
+        "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}",
+    ]
+    text = _run(cmd)
+    if verbose and text.strip():
+        print(text)
+    os.replace(tmp, out)
+    return out
+
+
+def build_all(force: bool = True, verbose: bool = False):
+    """libaops.so, then the extension module that links against it."""
+    lib = build_library(force=force, verbose=verbose)
+    ext = build_extension(force=force, verbose=verbose)
+    return lib, ext
+
+
 if __name__ == "__main__":
-    path = build_library(force="--force" in sys.argv, verbose=True)
-    print(path)
+    for path in build_all(force="--force" in sys.argv, verbose=True):
+        print(path)

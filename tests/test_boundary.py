@@ -8,6 +8,8 @@ import re
 import pytest
 import torch
 
+import cabi
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
@@ -18,18 +20,32 @@ def _declared_symbols():
 
 
 def test_library_loads_and_exports_every_declared_symbol():
-    import ascend910a_extras.ascend910a_extras_C as C
+    import ascend910a_extras
 
     declared = _declared_symbols()
-    assert len(declared) >= 11
-    lib = ctypes.CDLL(C.library_path())
+    assert len(declared) >= 25
+    assert ascend910a_extras.LIBRARY_PATH == cabi.LIBRARY
+    lib = ctypes.CDLL(ascend910a_extras.LIBRARY_PATH)
     for name in declared:
         assert hasattr(lib, name), f"libaops.so lacks {name}"
-    # the ctypes signature table covers exactly the declared functions
-    assert C.exported_symbols() == declared
-    assert C._lib.aops_version() >= 100
-    assert C._lib.aops_strerror(0) == b"success"
-    assert b"workspace" in C._lib.aops_strerror(-2)
+    # the test helper's signature table, parsed from the header, covers exactly the declared functions
+    assert sorted(cabi.declarations()) == declared
+    assert cabi.lib().aops_version() >= 200
+    assert cabi.lib().aops_strerror(0) == b"success"
+    assert b"workspace" in cabi.lib().aops_strerror(-2)
+
+
+def test_extension_module_mirrors_the_reference_binding():
+    """The product binds libaops.so from a compiled torch extension with the reference's module layout
+    (reference csrc/ffi/bind.cpp:53-61, csrc/ffi/ops.cpp:484-491): print_info at the top, the six operators
+    in the `ops` submodule."""
+    import ascend910a_extras.ascend910a_extras_C as C
+
+    assert C.__file__.endswith(".so")
+    assert C.library_version() == cabi.lib().aops_version()
+    for name in ("rope", "swiglu", "grouped_matmul", "add_rms_norm", "reshape_and_cache", "paged_attention"):
+        assert callable(getattr(C.ops, name))
+    assert callable(C.print_info)
 
 
 def test_api_surface_matches_reference_ops_py():
@@ -52,27 +68,23 @@ def test_api_surface_matches_reference_ops_py():
 
 
 def test_workspace_query_without_gpu():
-    import ascend910a_extras.ascend910a_extras_C as C
-
     # config 5 shape: 64 x 32 heads, 8 kv heads, D=128, P=128, 32 pages; one (max, sum, 128 floats)
     # record per (sequence, head, chunk), the number of chunks being the library's choice
     # plus one int per sequence
-    n = C._lib.aops_paged_attention_workspace(64, 32, 8, 128, 128, 32) - 64 * 4
+    n = cabi.lib().aops_paged_attention_workspace(64, 32, 8, 128, 128, 32) - 64 * 4
     per_chunk = 64 * 32 * 130 * 4
     assert n >= per_chunk and n % per_chunk == 0 and n // per_chunk <= 32
     # a single short sequence is split into more chunks than a large batch
-    n1 = C._lib.aops_paged_attention_workspace(1, 32, 8, 128, 128, 32) - 4
+    n1 = cabi.lib().aops_paged_attention_workspace(1, 32, 8, 128, 128, 32) - 4
     assert n1 // (32 * 130 * 4) > n // per_chunk
-    assert C._lib.aops_paged_attention_workspace(64, 32, 8, 100, 128, 32) == 0  # head_dim % 16 != 0
-    assert C._lib.aops_paged_attention_workspace(64, 32, 8, 512, 128, 32) == 0  # head_dim > 256
-    assert C._lib.aops_paged_attention_workspace(64, 32, 7, 128, 128, 32) == 0  # heads not a multiple of kv heads
-    assert C._lib.aops_paged_attention_workspace(64, 32, 8, 96, 24, 32) > 0     # generic kernel: token amount
+    assert cabi.lib().aops_paged_attention_workspace(64, 32, 8, 100, 128, 32) == 0  # head_dim % 16 != 0
+    assert cabi.lib().aops_paged_attention_workspace(64, 32, 8, 512, 128, 32) == 0  # head_dim > 256
+    assert cabi.lib().aops_paged_attention_workspace(64, 32, 7, 128, 128, 32) == 0  # heads not a multiple of kv heads
+    assert cabi.lib().aops_paged_attention_workspace(64, 32, 8, 96, 24, 32) > 0     # generic kernel: token amount
 
 
 def test_c_abi_rejects_bad_sizes_without_touching_the_gpu():
-    import ascend910a_extras.ascend910a_extras_C as C
-
-    lib = C._lib
+    lib = cabi.lib()
     assert lib.aops_swiglu_f16(None, None, 4, 12, None) == -1  # d % 8
     assert lib.aops_swiglu_f16(None, None, 4, 64, None) == -1  # null pointers
     assert lib.aops_swiglu_f16(None, None, 0, 64, None) == 0   # empty input is a no-op
@@ -92,6 +104,13 @@ def test_c_abi_rejects_bad_sizes_without_touching_the_gpu():
     assert lib.aops_matmul_nt_ws_f16(None, None, None, None, 0, 0, 64, 64, None) == 0
     assert lib.aops_matmul_nt_workspace(16, 100, 64) == 0                                   # invalid shape: no workspace
     assert lib.aops_grouped_matmul_f16(ctypes.c_void_p(8), ctypes.c_void_p(8), None, ctypes.c_void_p(8), 4, 64, 1, 64, None) == -1
+    assert lib.aops_grouped_matmul_variant_f16(0, None, None, None, None, 0, 64, 2, 64, None) == -1   # no such kernel
+    assert lib.aops_grouped_matmul_variant_f16(10, None, None, None, None, 0, 64, 2, 64, None) == -1
+    assert lib.aops_grouped_matmul_variant_f16(3, None, None, None, None, 0, 64, 2, 64, None) == 0
+    assert lib.aops_grouped_matmul_workspace(16, 100, 1, 64) == 0                                     # invalid shape
+    assert lib.aops_grouped_matmul_workspace(256, 14336, 2, 4096) == 0                                # only one expert is split over k
+    assert lib.aops_grouped_matmul_ws_f16(None, None, None, None, None, 0, 16, 100, 2, 64, None) == -1
+    assert lib.aops_grouped_matmul_ws_f16(None, None, None, None, None, 0, 0, 64, 2, 64, None) == 0
     # fused extensions
     assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 160, 2, 128, None) == -1   # k % 64
     assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 128, 2, 96, None) == -1    # n % 64
@@ -106,7 +125,7 @@ def test_c_abi_rejects_bad_sizes_without_touching_the_gpu():
     assert lib.aops_rope_reshape_and_cache_f16(*n, 2, 4, 2, 64, 8, 16, None) == -1                   # null pointers
     assert lib.aops_rope_reshape_and_cache_f16(*n, 0, 4, 2, 64, 8, 16, None) == 0
     m = [None] * 5 + [1e-6] + [None] * 8
-    assert lib.aops_qknorm_rope_reshape_and_cache_f16(*m, 2, 4, 2, 48, 8, 16, None) == -1            # 3 threads per head
+    assert lib.aops_qknorm_rope_reshape_and_cache_f16(*m, 2, 4, 2, 40, 8, 16, None) == -1            # head_dim % 16
     assert lib.aops_qknorm_rope_reshape_and_cache_f16(*m, 2, 4, 2, 64, 8, 16, None) == -1            # null pointers
     assert lib.aops_qknorm_rope_reshape_and_cache_f16(*m, 0, 4, 2, 64, 8, 16, None) == 0
 
@@ -173,12 +192,12 @@ def test_misaligned_fp16_views_are_refused():
     import ascend910a_extras.ascend910a_extras_C as C
 
     flat = torch.zeros(4 * 64 + 4, dtype=H)
-    assert C._ptr(flat[:256].view(4, 64)) == flat.data_ptr()
+    assert C.tensor_address(flat[:256].view(4, 64)) == flat.data_ptr()
     with pytest.raises(RuntimeError, match="16-byte aligned"):
-        C._ptr(flat[4:260].view(4, 64))
+        C.tensor_address(flat[4:260].view(4, 64))
     ids = torch.zeros(9, dtype=torch.int32)
-    assert C._ptr(ids[1:]) == ids.data_ptr() + 4
-    assert C._ptr(flat[:0]) is None
+    assert C.tensor_address(ids[1:]) == ids.data_ptr() + 4
+    assert C.tensor_address(flat[:0]) == 0
 
 
 def test_product_package_does_not_import_the_oracle():
