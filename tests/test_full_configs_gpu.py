@@ -95,13 +95,110 @@ def test_config4_moe_grouped_matmul(ops, dev):
     yp = ops.grouped_matmul(xp.to(dev), wd.transpose(1, 2), gd).cpu()
     assert torch.equal(yp[s:t], yc[s:t][perm])
     assert torch.equal(yp[:s], yc[:s]) and torch.equal(yp[t:], yc[t:])
-    # the second GEMM of the expert MLP against the oracle end to end on one expert
+    # the second GEMM of the expert MLP (K = 768, N = 2048) against the oracle on the first, second, a middle
+    # and the last expert, with the device's own activation as input ...
     hgu = ops.swiglu(y)
+    hc = hgu.cpu()
     w2 = (0.02 * torch.randn(E, hidden, inter)).half()
-    out = ops.grouped_matmul(hgu, w2.to(dev).transpose(1, 2), gd).cpu()
+    w2d = w2.to(dev)
+    out = ops.grouped_matmul(hgu, w2d.transpose(1, 2), gd)
+    outc = out.cpu()
+    for e in (0, 1, 63, 127):
+        s, t = bounds[e], bounds[e + 1]
+        torch.testing.assert_close(hc[s:t].float(), R.swiglu_ref(yc[s:t]).float(), rtol=1e-2, atol=1e-2)
+        ref = (hc[s:t].float() @ w2[e].float().T).half()
+        torch.testing.assert_close(outc[s:t].float(), ref.float(), rtol=2e-2, atol=2e-2)
+    # ... and end to end (oracle activation of the oracle's gate_up) on one expert
     s, t = bounds[127], bounds[128]
-    ref = (R.swiglu_ref(yc[s:t]).float() @ w2[127].float().T).half()
-    torch.testing.assert_close(out[s:t].float(), ref.float(), rtol=2e-2, atol=2e-2)
+    ref = R.grouped_matmul_ref(R.swiglu_ref(R.grouped_matmul_ref(x[s:t], w1[127:128].transpose(1, 2), torch.tensor([t - s]))),
+                               w2[127:128].transpose(1, 2), torch.tensor([t - s]))
+    torch.testing.assert_close(outc[s:t].float(), ref.float(), rtol=2e-2, atol=2e-2)
+    # the same size-independent properties for the down projection, over all 32768 rows
+    out2 = ops.grouped_matmul(hgu * 2, w2d.transpose(1, 2), gd)
+    normal = out.abs() >= 2.0 ** -13
+    assert torch.equal(out2[normal], (out * 2)[normal])
+    e = 77
+    s, t = bounds[e], bounds[e + 1]
+    perm = torch.randperm(t - s)
+    hp = hc.clone(); hp[s:t] = hc[s:t][perm]
+    outp = ops.grouped_matmul(hp.to(dev), w2d.transpose(1, 2), gd).cpu()
+    assert torch.equal(outp[s:t], outc[s:t][perm])
+    assert torch.equal(outp[:s], outc[:s]) and torch.equal(outp[t:], outc[t:])
+
+
+def test_config4_every_expert_against_the_oracle(ops, dev):
+    """Config 4 at full size, both projections, compared with the fp32 oracle on a seeded sample of rows from
+    every one of the 128 experts (first row, last row and up to six more of each group: the rows where a
+    scheduler or tile-boundary mistake would show)."""
+    torch.manual_seed(1)
+    E, hidden, inter, rows = 128, 2048, 768, 4096 * 8
+    ids = torch.randint(0, E, (rows,))
+    gl = R.make_group_list(ids, E)
+    bounds = [0] + gl.tolist()
+    x = torch.randn(rows, hidden).half()
+    w1 = (0.02 * torch.randn(E, 2 * inter, hidden)).half()
+    w2 = (0.02 * torch.randn(E, hidden, inter)).half()
+    xd, gd = x.to(dev), gl.to(dev)
+    y = ops.grouped_matmul(xd, w1.to(dev).transpose(1, 2), gd)
+    h = ops.swiglu(y)
+    out = ops.grouped_matmul(h, w2.to(dev).transpose(1, 2), gd)
+    yc, hc, outc = y.cpu(), h.cpu(), out.cpu()
+    g = torch.Generator().manual_seed(2)
+    for e in range(E):
+        s, t = bounds[e], bounds[e + 1]
+        if t == s:
+            continue
+        pick = torch.unique(torch.cat([torch.tensor([s, t - 1]), s + torch.randint(0, t - s, (6,), generator=g)]))
+        ref1 = x[pick].float() @ w1[e].float().T
+        torch.testing.assert_close(yc[pick].float(), ref1, rtol=2e-2, atol=2e-2)
+        ref2 = hc[pick].float() @ w2[e].float().T
+        torch.testing.assert_close(outc[pick].float(), ref2, rtol=2e-2, atol=2e-2)
+
+
+def test_config4_fused_gate_up_against_the_oracle(ops, dev):
+    """The fused forms of config 4's gate_up projection at full size (K = 2048, N = 1536, 128 experts, 32768 routed
+    rows) against the oracle chain swiglu_ref(grouped_matmul_ref(...)), not against the device's own chain:
+    `fused.grouped_matmul_swiglu` on the expert-sorted rows and `grouped_matmul_swiglu_gather` on the token-order
+    rows with the routing's sorted index, on sampled experts (whole groups) plus sampled rows of every expert."""
+    import ascend910a_extras.ascend910a_extras_C as C
+    import ascend910a_extras.fused as fused
+    import ascend910a_extras.moe as moe
+
+    torch.manual_seed(3)
+    E, hidden, inter, tokens, topk = 128, 2048, 768, 4096, 8
+    topk_ids = torch.randint(0, E, (tokens, topk), dtype=torch.int32)
+    x = torch.randn(tokens, hidden).half()
+    w1 = (0.02 * torch.randn(E, 2 * inter, hidden)).half()
+    xd, w1d = x.to(dev), w1.to(dev)
+    sorted_idx, _, gl = moe.moe_sort(topk_ids.to(dev), E)
+    # the routing itself against the oracle's construction (benchmark/test_grouped_matmul.py:46-50)
+    order_ref, _, gl_ref = R.moe_sort_ref(topk_ids, E)
+    assert torch.equal(sorted_idx.cpu(), order_ref.int()) and torch.equal(gl.cpu(), gl_ref)
+    bounds = [0] + gl_ref.tolist()
+    src = (order_ref // topk).long()                 # token of every sorted row
+    xs = x[src]                                      # expert-sorted activations, built on the host
+    a_sorted = fused.grouped_matmul_swiglu(xs.to(dev), w1d.transpose(1, 2), gl).cpu()
+    a_gather = C.grouped_matmul_swiglu_gather(xd, sorted_idx, topk, w1d.transpose(1, 2), gl).cpu()
+    assert a_sorted.shape == (tokens * topk, inter)
+
+    def oracle(rows_idx, e):
+        n = len(rows_idx)
+        return R.swiglu_ref(R.grouped_matmul_ref(xs[rows_idx], w1[e:e + 1].transpose(1, 2), torch.tensor([n])))
+
+    for e in (0, 1, 64, 127):                         # whole groups
+        s, t = bounds[e], bounds[e + 1]
+        ref = oracle(torch.arange(s, t), e).float()
+        torch.testing.assert_close(a_sorted[s:t].float(), ref, rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(a_gather[s:t].float(), ref, rtol=2e-2, atol=2e-2)
+    g = torch.Generator().manual_seed(4)
+    for e in range(E):                                # first, last and four more rows of every expert
+        s, t = bounds[e], bounds[e + 1]
+        if t == s:
+            continue
+        pick = torch.unique(torch.cat([torch.tensor([s, t - 1]), s + torch.randint(0, t - s, (4,), generator=g)]))
+        ref = oracle(pick, e).float()
+        torch.testing.assert_close(a_sorted[pick].float(), ref, rtol=2e-2, atol=2e-2)
+        torch.testing.assert_close(a_gather[pick].float(), ref, rtol=2e-2, atol=2e-2)
 
 
 def test_config5_decode_attention_with_rope(ops, dev):

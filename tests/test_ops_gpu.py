@@ -8,6 +8,7 @@ import math
 import pytest
 import torch
 
+import cabi
 import oracle.ops_ref as R
 
 pytestmark = pytest.mark.gpu
@@ -206,7 +207,10 @@ def test_rope_reshape_and_cache_fused_equals_the_chain(ops, dev, B, Hq, Hkv, D, 
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,D,NB,P", [(64, 32, 8, 128, 2304, 128), (5, 6, 2, 64, 7, 16), (3, 1, 1, 16, 4, 8), (9, 4, 4, 256, 9, 32), (7, 3, 1, 32, 5, 4),
-                                             (1200, 4, 4, 64, 80, 16)])
+                                             (1200, 4, 4, 64, 80, 16),
+                                             # head sizes whose threads per head are no power of two: 3, 5, 6, 7, 10, 12 and 20 threads
+                                             (37, 5, 1, 48, 9, 16), (300, 7, 3, 80, 40, 8), (11, 4, 2, 96, 5, 16), (5, 3, 1, 112, 4, 4),
+                                             (19, 9, 3, 160, 7, 16), (64, 16, 4, 192, 20, 32), (3, 2, 2, 320, 3, 16)])
 def test_qknorm_rope_reshape_and_cache_fused(ops, dev, B, Hq, Hkv, D, NB, P):
     """Per-head RMSNorm of q and k + rope + cache write in one launch, against the oracle (RMSNorm rounded to fp16,
     then rotated) and against the chain of separate device operators where those take the shape."""
@@ -297,11 +301,10 @@ def test_grouped_matmul_reference_script_shape(ops, dev):
 
 def test_grouped_matmul_does_not_write_past_the_last_group(ops, dev):
     x, w, gl = _gmm_case(256, 128, 128, 2, seed=3, counts=[50, 60])
-    import ascend910a_extras.ascend910a_extras_C as C
     y = torch.full((256, 128), 5.0, dtype=H, device=dev)
     xd, wd, gd = x.to(dev), w.to(dev), gl.to(dev)
-    code = C._lib.aops_grouped_matmul_f16(xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y.data_ptr(), 256, 128, 2, 128,
-                                          torch.cuda.current_stream().cuda_stream)
+    code = cabi.lib().aops_grouped_matmul_f16(xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y.data_ptr(), 256, 128, 2, 128,
+                                          cabi.stream(dev))
     assert code == 0
     assert torch.all(y[110:] == 5.0)
     ref = R.grouped_matmul_ref(x, w, gl)
@@ -318,17 +321,15 @@ def test_grouped_matmul_does_not_write_past_the_last_group(ops, dev):
         (321, 256, 64, 1, [321]),                         # one expert, one row past a full tile, minimum N
     ],
 )
-def test_grouped_matmul_every_kernel(ops, dev, monkeypatch, variant, rows, K, N, E, counts):
-    """The tile shape / kernel is normally chosen from the problem size; AOPS_GMM_VARIANT forces one,
-    so that every kernel sees the edge cases (6 = persistent kernel, needs K % 128 == 0, K >= 256; 7, 8 = direct-copy kernels with smaller tiles)."""
-    import ascend910a_extras.ascend910a_extras_C as C
-    monkeypatch.setenv("AOPS_GMM_VARIANT", str(variant))
+def test_grouped_matmul_every_kernel(ops, dev, variant, rows, K, N, E, counts):
+    """The tile shape / kernel is normally chosen from the problem size; aops_grouped_matmul_variant_f16 fixes
+    one, so that every kernel sees the edge cases (6 = persistent kernel, needs K % 128 == 0, K >= 256; 7, 8 = direct-copy kernels with smaller tiles)."""
     x, w, gl = _gmm_case(rows, K, N, E, seed=variant, counts=counts)
     end = int(gl[-1])
     y = torch.full((rows, N), 5.0, dtype=H, device=dev)
     xd, wd, gd = x.to(dev), w.transpose(1, 2).contiguous().to(dev), gl.to(dev)   # storage [E, N, K]
-    code = C._lib.aops_grouped_matmul_f16(xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y.data_ptr(), rows, K, E, N,
-                                          torch.cuda.current_stream().cuda_stream)
+    code = cabi.lib().aops_grouped_matmul_variant_f16(variant, xd.data_ptr(), wd.data_ptr(), gd.data_ptr(),
+                                                      y.data_ptr(), rows, K, E, N, cabi.stream(dev))
     assert code == 0
     ref = R.grouped_matmul_ref(x, w, gl)
     torch.testing.assert_close(y.cpu()[:end].float(), ref[:end].float(), **GMM_TOL)
@@ -386,20 +387,18 @@ SPLIT_K_SHAPES = [(256, 14336, 4096), (16, 8192, 1024), (300, 4096, 256), (1, 20
 def test_matmul_nt_split_k(ops, dev, m, k, n):
     """Few rows and a long k: the k range is split over workgroups and a second kernel adds the partial results.
     Against the fp32 product, against the whole-k kernels, and bit-identical from call to call."""
-    import ascend910a_extras.ascend910a_extras_C as C
-
     g = _gen(m + k + n)
     x = torch.randn(m, k, generator=g).half()
     w = (torch.randn(n, k, generator=g) / k ** 0.5).half()
     xd, wd = x.to(dev), w.to(dev)
-    ws_bytes = C._lib.aops_matmul_nt_workspace(m, k, n)
+    ws_bytes = cabi.lib().aops_matmul_nt_workspace(m, k, n)
     assert ws_bytes > 0, "the shape is meant to take the split-k path"
     y = ops.matmul(xd, wd)
     ref = x.float() @ w.float().T
     torch.testing.assert_close(y.cpu().float(), ref, **GMM_TOL)
     # the whole-k kernel (no workspace) agrees to rounding: both accumulate in fp32, in a different order
     whole = torch.empty_like(y)
-    assert C._lib.aops_matmul_nt_f16(xd.data_ptr(), wd.data_ptr(), whole.data_ptr(), m, k, n, C._stream(dev)) == 0
+    assert cabi.lib().aops_matmul_nt_f16(xd.data_ptr(), wd.data_ptr(), whole.data_ptr(), m, k, n, cabi.stream(dev)) == 0
     torch.testing.assert_close(y.float(), whole.float(), rtol=2e-3, atol=2e-3)
     assert torch.equal(ops.matmul(xd, wd), y)
     # one expert through the grouped entry of the Python API takes the same path
@@ -408,8 +407,8 @@ def test_matmul_nt_split_k(ops, dev, m, k, n):
     # a workspace that is too small is refused, the output untouched
     small = torch.empty(ws_bytes - 1, dtype=torch.uint8, device=dev)
     out = torch.zeros_like(y)
-    code = C._lib.aops_matmul_nt_ws_f16(xd.data_ptr(), wd.data_ptr(), out.data_ptr(), small.data_ptr(), ws_bytes - 1,
-                                        m, k, n, C._stream(dev))
+    code = cabi.lib().aops_matmul_nt_ws_f16(xd.data_ptr(), wd.data_ptr(), out.data_ptr(), small.data_ptr(), ws_bytes - 1,
+                                        m, k, n, cabi.stream(dev))
     torch.cuda.synchronize()
     assert code == -2 and not out.any()
 
@@ -419,49 +418,74 @@ FEW_ROWS_SHAPES = [(1, 4096, 4096), (16, 512, 2048), (7, 576, 2048), (16, 14336,
 
 
 @pytest.mark.parametrize("m,k,n", FEW_ROWS_SHAPES)
-def test_matmul_nt_few_rows(ops, dev, m, k, n, monkeypatch):
+def test_matmul_nt_few_rows(ops, dev, m, k, n):
     """At most 16 rows (the projections of a small decode batch): one workgroup per 16 rows of W, every wave
     copies its own pieces of W and x into LDS and waits for them alone, no workspace.  Against the fp32 product,
     against the tile kernels, bit-identical from call to call; through the grouped entry the rows past
     group_list[0] stay untouched.  k with a short last piece, n that is not a multiple of the XCD run."""
-    import ascend910a_extras.ascend910a_extras_C as C
-
     g = _gen(m + k + n)
     x = torch.randn(m, k, generator=g).half()
     w = (torch.randn(n, k, generator=g) / k ** 0.5).half()
     xd, wd = x.to(dev), w.to(dev)
-    assert C._lib.aops_matmul_nt_workspace(m, k, n) == 0
+    assert cabi.lib().aops_matmul_nt_workspace(m, k, n) == 0
     y = ops.matmul(xd, wd)
     ref = x.float() @ w.float().T
     torch.testing.assert_close(y.cpu().float(), ref, **GMM_TOL)
     assert torch.equal(ops.matmul(xd, wd), y)
-    monkeypatch.setenv("AOPS_GMM_VARIANT", "5")          # the 64 x 64 tile kernel on the same product
-    tiles = ops.matmul(xd, wd)
-    monkeypatch.delenv("AOPS_GMM_VARIANT")
+    tiles = torch.empty_like(y)                          # the 64 x 64 tile kernel on the same product
+    assert cabi.lib().aops_grouped_matmul_variant_f16(5, xd.data_ptr(), wd.data_ptr(), None, tiles.data_ptr(), m, k, 1, n,
+                                                      cabi.stream(dev)) == 0
     torch.testing.assert_close(y.float(), tiles.float(), rtol=2e-3, atol=2e-3)
     # one group that ends before the last row: later rows are not written
     part = max(m - 3, 0)
     gl = torch.tensor([part], dtype=torch.int64, device=dev)
     out = torch.full((m, n), 7.0, dtype=H, device=dev)
-    code = C._lib.aops_grouped_matmul_f16(xd.data_ptr(), wd.data_ptr(), gl.data_ptr(), out.data_ptr(), m, k, 1, n,
-                                          C._stream(dev))
+    code = cabi.lib().aops_grouped_matmul_f16(xd.data_ptr(), wd.data_ptr(), gl.data_ptr(), out.data_ptr(), m, k, 1, n,
+                                          cabi.stream(dev))
     torch.cuda.synchronize()
     assert code == 0
     assert torch.equal(out[:part], y[:part]) and bool((out[part:] == 7.0).all())
 
 
+@pytest.mark.parametrize("m,k,n,part", [(256, 14336, 4096, 200), (64, 4096, 1024, 1), (100, 2048, 512, 0), (128, 8192, 256, 128)])
+def test_grouped_matmul_one_expert_split_k_honours_group_list(ops, dev, m, k, n, part):
+    """One expert, few rows, long k: the library splits the k range (two kernels, workspace).  Rows at or past
+    group_list[0] must stay unwritten there too, as in every other kernel."""
+    assert cabi.lib().aops_grouped_matmul_workspace(m, k, 1, n) > 0          # the shape does take the split path
+    assert cabi.lib().aops_grouped_matmul_workspace(m, k, 1, n) == cabi.lib().aops_matmul_nt_workspace(m, k, n)
+    g = _gen(m + part)
+    x = torch.randn(m, k, generator=g).half()
+    w = (torch.randn(1, n, k, generator=g) / k ** 0.5).half()
+    gl = torch.tensor([part], dtype=torch.int64)
+    xd, wd, gd = x.to(dev), w.to(dev), gl.to(dev)
+    ws_bytes = cabi.lib().aops_grouped_matmul_workspace(m, k, 1, n)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    y = torch.full((m, n), 7.0, dtype=H, device=dev)
+    code = cabi.lib().aops_grouped_matmul_ws_f16(xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y.data_ptr(), ws.data_ptr(),
+                                                 ws_bytes, m, k, 1, n, cabi.stream(dev))
+    assert code == 0
+    torch.cuda.synchronize()
+    assert bool((y[part:] == 7.0).all())
+    ref = x.float() @ w[0].float().T
+    torch.testing.assert_close(y[:part].cpu().float(), ref[:part], **GMM_TOL)
+    # the Python API takes the same path; its fresh output holds the same rows
+    y_api = ops.grouped_matmul(xd, wd.transpose(1, 2), gd)
+    assert torch.equal(y_api[:part], y[:part])
+    # a workspace that is wanted but too small is refused
+    assert cabi.lib().aops_grouped_matmul_ws_f16(xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y.data_ptr(), ws.data_ptr(),
+                                                 ws_bytes - 1, m, k, 1, n, cabi.stream(dev)) == -2
+
+
 def test_matmul_nt_ws_without_split(ops, dev):
     """Shapes with enough output tiles need no workspace; the workspace entry point then equals the plain one."""
-    import ascend910a_extras.ascend910a_extras_C as C
-
     m, k, n = 512, 512, 8192
-    assert C._lib.aops_matmul_nt_workspace(m, k, n) == 0
+    assert cabi.lib().aops_matmul_nt_workspace(m, k, n) == 0
     g = _gen(5)
     x = torch.randn(m, k, generator=g).half().to(dev)
     w = (torch.randn(n, k, generator=g) / k ** 0.5).half().to(dev)
     a, b = torch.empty(m, n, dtype=H, device=dev), torch.empty(m, n, dtype=H, device=dev)
-    assert C._lib.aops_matmul_nt_ws_f16(x.data_ptr(), w.data_ptr(), a.data_ptr(), None, 0, m, k, n, C._stream(dev)) == 0
-    assert C._lib.aops_matmul_nt_f16(x.data_ptr(), w.data_ptr(), b.data_ptr(), m, k, n, C._stream(dev)) == 0
+    assert cabi.lib().aops_matmul_nt_ws_f16(x.data_ptr(), w.data_ptr(), a.data_ptr(), None, 0, m, k, n, cabi.stream(dev)) == 0
+    assert cabi.lib().aops_matmul_nt_f16(x.data_ptr(), w.data_ptr(), b.data_ptr(), m, k, n, cabi.stream(dev)) == 0
     assert torch.equal(a, b)
 
 
@@ -636,6 +660,10 @@ def test_paged_attention_batch_larger_than_a_wave(ops, dev, B, Hq, Hkv, P):
         (2, 32, 2, 128, 64, [100, 1000]),       # 16 query heads per kv head (matrix-core path)
         (2, 8, 2, 128, 24, [25, 300]),          # block size not a multiple of 32
         (1, 5, 5, 48, 8, [77]),                 # head_dim 48
+        (2, 32, 1, 64, 16, [70, 300]),          # more than 16 query heads per kv head: generic kernel
+        (2, 24, 1, 64, 32, [33, 129]),
+        (3, 17, 1, 64, 16, [1, 16, 250]),
+        (2, 40, 2, 128, 16, [100, 37]),         # 20 heads per kv head at head_dim 128
     ],
 )
 def test_paged_attention_other_shapes(ops, dev, B, Hq, Hkv, D, P, lens):
@@ -665,9 +693,7 @@ def test_paged_attention_other_shapes(ops, dev, B, Hq, Hkv, D, P, lens):
 def test_paged_attention_matrix_core_path_any_group_and_page_size(ops, dev, B, Hq, Hkv, P, lens):
     """head_dim 128 takes the matrix-core kernel for every group size up to 16 and every page size that is a multiple
     of 16; unused cache slots hold NaN and unused table entries -1."""
-    import ascend910a_extras.ascend910a_extras_C as C
-
-    assert C._lib.aops_paged_attention_workspace(B, Hq, Hkv, 128, P, 64) > 16   # not the generic kernel
+    assert cabi.lib().aops_paged_attention_workspace(B, Hq, Hkv, 128, P, 64) > 16   # not the generic kernel
     case = _paged_case(B, Hq, Hkv, 128, P, lens, seed=9, poison=True)
     o = _run_pa(ops, dev, case)
     ref = R.paged_attention_ref(*case)
@@ -688,9 +714,7 @@ def test_paged_attention_matrix_core_path_any_group_and_page_size(ops, dev, B, H
     ],
 )
 def test_paged_attention_matrix_core_path_other_head_sizes(ops, dev, B, Hq, Hkv, D, P, lens):
-    import ascend910a_extras.ascend910a_extras_C as C
-
-    assert C._lib.aops_paged_attention_workspace(B, Hq, Hkv, D, P, 64) > 16   # not the generic kernel
+    assert cabi.lib().aops_paged_attention_workspace(B, Hq, Hkv, D, P, 64) > 16   # not the generic kernel
     case = _paged_case(B, Hq, Hkv, D, P, lens, seed=13, poison=True)
     o = _run_pa(ops, dev, case)
     ref = R.paged_attention_ref(*case)
@@ -730,6 +754,16 @@ def test_paged_attention_balanced_partition(ops, dev, B, Hq, Hkv, P, maxlen, see
     assert (o.float() - ref.float()).abs().max() < 3e-3
     # deterministic: the partial results are merged in a fixed order
     assert torch.equal(_run_pa(ops, dev, case), o)
+
+
+def test_paged_attention_wide_groups_take_the_generic_kernel():
+    """The matrix-core kernel holds one of at most 16 query heads of a kv head per lane (8 at head_dim 256);
+    wider groups must be routed to the generic kernel, which needs no workspace (the query answers 16)."""
+    ws = cabi.lib().aops_paged_attention_workspace
+    for hq, hkv, d in [(32, 1, 64), (24, 1, 64), (17, 1, 64), (40, 2, 128), (9, 1, 256)]:
+        assert ws(2, hq, hkv, d, 16, 64) == 16
+    for hq, hkv, d in [(16, 1, 64), (32, 2, 128), (8, 1, 256)]:
+        assert ws(2, hq, hkv, d, 16, 64) > 16
 
 
 def test_paged_attention_very_long_context(ops, dev):
