@@ -1,14 +1,17 @@
 #!/usr/bin/env python3
 """Benchmark of the ascend910a_extras operator set on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|pa|gmm|...] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|norm|cache|rope|mlp|moe|pa_more|dense|scaled,...] [--no-cpu]
 
 A "step" is one paged_attention decode call over the batch of BASELINE.json configs[4]
 (64 sequences, 32 query / 8 kv heads, head_dim 128, contexts ~U[512, 4096], block 128): the
 largest HBM-bound workload of the operator set and the one the printed `value` is quoted on.
-Every other configuration is measured as well and reported under `per_op` of the same JSON line
-(add_rms_norm, reshape_and_cache, swiglu and the two dense GEMMs of the MLP, the MoE grouped GEMMs,
-rope, plus clearly labelled scaled shapes of the small operators).
+Every other configuration is measured as well (add_rms_norm, reshape_and_cache, swiglu and the two
+dense GEMMs of the MLP, the MoE grouped GEMMs, rope, further paged-attention batches, a compute-bound
+dense product, plus clearly labelled scaled shapes of the small operators): the full records go out as
+one `{"per_op": [...]}` JSON line BEFORE the headline, and a compact list of them
+(`roofline.per_kernel`: operator, config, microseconds, fraction of the bounding peak, CPU ms) sits inside
+the headline, which is the last line printed.
 
 Timing:
   * `ms_per_step` / `value`: wall clock around exactly K eager steps through the Python API,
@@ -19,13 +22,16 @@ Timing:
     sized so that the footprint between two uses of the same buffer exceeds the 256 MB Infinity
     Cache.  Algorithmic bytes = every input read once, every output written once.
   * `cpu_baseline` / `per_op[*].cpu_ms`: the CPU oracle (plain torch, fp32 math) on the same
-    inputs on this machine's host cores, median of a few runs.  The oracle is the checker and
-    the timed baseline only; nothing measured on the GPU goes through it.
+    inputs on this machine's host cores: one warm-up run, then the median of three timed runs.
+    The oracle is the checker and the timed baseline only; nothing measured on the GPU goes
+    through it.
+  * `launch_floor_us`: an empty kernel with the operator's launch geometry through the same
+    graph-replay timer: what a latency-bound operator is up against besides HBM.
 """
 from __future__ import annotations
 
 import argparse
-import ctypes
+import hashlib
 import json
 import math
 import os
@@ -34,7 +40,7 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for _p in (ROOT, os.path.join(ROOT, "ascend-ops_amd")):
+for _p in (ROOT, os.path.join(ROOT, "ascend-ops_amd"), os.path.join(ROOT, "tests")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
@@ -98,14 +104,18 @@ def time_eager(calls, warmup, iters):
     return ms * 1e3 / iters
 
 
-def time_cpu(fn, runs=3):
-    fn()
+CPU_RUNS = 3
+
+
+def time_cpu(fn, runs=CPU_RUNS):
+    """One warm-up run, then the median of `runs` timed ones (milliseconds); returns (ms, last result)."""
+    out = fn()
     ts = []
     for _ in range(runs):
         t0 = time.perf_counter()
-        fn()
+        out = fn()
         ts.append(time.perf_counter() - t0)
-    return statistics.median(ts) * 1e3
+    return statistics.median(ts) * 1e3, out
 
 
 def n_sets_for(bytes_per_set, lo=2, hi=128):
@@ -118,9 +128,9 @@ class Lib:
 
     def __init__(self):
         import torch
-        import ascend910a_extras.ascend910a_extras_C as C
+        import cabi  # tests/cabi.py: libaops.so through ctypes, signatures parsed from include/aops.h
 
-        self.lib = C._lib
+        self.lib = cabi.lib()
         self.torch = torch
 
     def stream(self):
@@ -129,6 +139,11 @@ class Lib:
     def check(self, code):
         if code != 0:
             raise RuntimeError(self.lib.aops_strerror(code).decode())
+
+    def launch_floor_us(self, workgroups, threads):
+        """Per-launch time of an empty kernel with this geometry, through the timer the operators use."""
+        med, _ = time_graph([lambda: self.check(self.lib.aops_empty_launch(workgroups, threads, self.stream()))])
+        return round(med, 3)
 
 
 def entry(op, config, shape, bound, alg_bytes, alg_flops, gpu_us, gpu_us_min, eager_us, cpu_ms, cores, note=None):
@@ -148,6 +163,7 @@ def entry(op, config, shape, bound, alg_bytes, alg_flops, gpu_us, gpu_us_min, ea
     if cpu_ms is not None:
         e["cpu_ms"] = round(cpu_ms, 3)
         e["cpu_cores"] = cores
+        e["cpu_runs"] = f"1 warm-up + median of {CPU_RUNS}"
         e["gpu_over_cpu"] = round(cpu_ms * 1e3 / gpu_us, 1)
     if note:
         e["note"] = note
@@ -155,7 +171,7 @@ def entry(op, config, shape, bound, alg_bytes, alg_flops, gpu_us, gpu_us_min, ea
 
 
 # --------------------------------------------------------------------------------------- workloads
-def bench_add_rms_norm(L, ops, R, dev, cpu, T, config, note=None):
+def bench_add_rms_norm(L, ops, R, dev, cpu, T, config, note=None, floor=False):
     import torch
 
     Hd, eps = 4096, 1e-6
@@ -181,12 +197,15 @@ def bench_add_rms_norm(L, ops, R, dev, cpu, T, config, note=None):
     y_ref, res_ref = R.add_rms_norm_ref(x, r, w, eps)
     torch.testing.assert_close(ys[-1].cpu().float(), y_ref.float(), rtol=1e-2, atol=1e-2)
     assert torch.equal(os_[-1].cpu(), res_ref)
-    cpu_ms = time_cpu(lambda: R.add_rms_norm_ref(x, r, w, eps)) if cpu else None
-    return entry("add_rms_norm", config, f"x,residual [{T},{Hd}] f16", "hbm", alg, 0, med, mn, eager, cpu_ms,
-                 torch.get_num_threads(), note)
+    cpu_ms = time_cpu(lambda: R.add_rms_norm_ref(x, r, w, eps))[0] if cpu else None
+    e = entry("add_rms_norm", config, f"x,residual [{T},{Hd}] f16", "hbm", alg, 0, med, mn, eager, cpu_ms,
+              torch.get_num_threads(), note)
+    if floor:
+        e["launch_floor_us"] = L.launch_floor_us(T, 512)  # one workgroup of 512 threads per row
+    return e
 
 
-def bench_swiglu(L, ops, R, dev, cpu, T, d, config, note=None):
+def bench_swiglu(L, ops, R, dev, cpu, T, d, config, note=None, floor=False):
     import torch
 
     torch.manual_seed(0)
@@ -202,12 +221,15 @@ def bench_swiglu(L, ops, R, dev, cpu, T, d, config, note=None):
     med, mn = time_graph([mk(i) for i in range(n)])
     eager = time_eager([(lambda i=i: ops.swiglu(xs[i])) for i in range(n)], 10, 100)
     torch.testing.assert_close(ys[-1].cpu().float(), R.swiglu_ref(x).float(), rtol=1e-2, atol=1e-2)
-    cpu_ms = time_cpu(lambda: R.swiglu_ref(x)) if cpu else None
-    return entry("swiglu", config, f"x [{T},{2 * d}] f16", "hbm", alg, 0, med, mn, eager, cpu_ms,
-                 torch.get_num_threads(), note)
+    cpu_ms = time_cpu(lambda: R.swiglu_ref(x))[0] if cpu else None
+    e = entry("swiglu", config, f"x [{T},{2 * d}] f16", "hbm", alg, 0, med, mn, eager, cpu_ms,
+              torch.get_num_threads(), note)
+    if floor:
+        e["launch_floor_us"] = L.launch_floor_us((T * d // 8 + 511) // 512, 256)  # 2 x 16 bytes of output per thread
+    return e
 
 
-def bench_rope(L, ops, R, dev, cpu, B, config, note=None):
+def bench_rope(L, ops, R, dev, cpu, B, config, note=None, floor=False):
     import torch
 
     Hq, Hkv, D, max_pos = 32, 8, 128, 4096
@@ -234,12 +256,15 @@ def bench_rope(L, ops, R, dev, cpu, B, config, note=None):
     rq, rk = R.rope_ref(q, k, pos, cos, sin)
     torch.testing.assert_close(oq[-1].cpu().float(), rq.float(), rtol=1e-2, atol=1e-2)
     torch.testing.assert_close(ok[-1].cpu().float(), rk.float(), rtol=1e-2, atol=1e-2)
-    cpu_ms = time_cpu(lambda: R.rope_ref(q, k, pos, cos, sin)) if cpu else None
-    return entry("rope", config, f"q [{B},{Hq},{D}], k [{B},{Hkv},{D}] f16", "hbm", alg, 0, med, mn, eager, cpu_ms,
-                 torch.get_num_threads(), note)
+    cpu_ms = time_cpu(lambda: R.rope_ref(q, k, pos, cos, sin))[0] if cpu else None
+    e = entry("rope", config, f"q [{B},{Hq},{D}], k [{B},{Hkv},{D}] f16", "hbm", alg, 0, med, mn, eager, cpu_ms,
+              torch.get_num_threads(), note)
+    if floor:
+        e["launch_floor_us"] = L.launch_floor_us((B * (Hq + Hkv) * D // 16 + 255) // 256, 256)  # 8 pairs per thread
+    return e
 
 
-def bench_reshape_and_cache(L, ops, R, dev, cpu, T, config, note=None, consecutive=False):
+def bench_reshape_and_cache(L, ops, R, dev, cpu, T, config, note=None, consecutive=False, floor=False):
     import torch
 
     Hkv, D, NB, P = 8, 128, 1024, 128
@@ -273,12 +298,15 @@ def bench_reshape_and_cache(L, ops, R, dev, cpu, T, config, note=None, consecuti
     vc_ref = torch.zeros_like(kc_ref)
     cpu_ms = None
     if cpu:
-        cpu_ms = time_cpu(lambda: R.reshape_and_cache_ref(key, kc_ref, slots, value, vc_ref), runs=2 if T > 4096 else 3)
+        cpu_ms = time_cpu(lambda: R.reshape_and_cache_ref(key, kc_ref, slots, value, vc_ref))[0]
     else:
         R.reshape_and_cache_ref(key, kc_ref, slots, value, vc_ref)
     assert torch.equal(kcs[0].cpu(), kc_ref) and torch.equal(vcs[0].cpu(), vc_ref), "reshape_and_cache not bit-exact"
-    return entry("reshape_and_cache", config, f"key,value [{T},{Hkv},{D}] -> caches [{NB},{Hkv * D // 16},{P},16] f16",
-                 "hbm", alg, 0, med, mn, eager, cpu_ms, torch.get_num_threads(), note)
+    e = entry("reshape_and_cache", config, f"key,value [{T},{Hkv},{D}] -> caches [{NB},{Hkv * D // 16},{P},16] f16",
+              "hbm", alg, 0, med, mn, eager, cpu_ms, torch.get_num_threads(), note)
+    if floor:
+        e["launch_floor_us"] = L.launch_floor_us(2 * ((T * Hkv * D // 8 + 255) // 256), 256)  # 16 bytes per thread, K and V
+    return e
 
 
 def _gmm_entry(L, ops, R, dev, cpu, op, config, x, w_storage, gl, note=None, check_rows=4096):
@@ -296,16 +324,14 @@ def _gmm_entry(L, ops, R, dev, cpu, op, config, x, w_storage, gl, note=None, che
     ws = [wd] + [wd.clone() for _ in range(n - 1)]
     ys = [torch.empty(rows, N, dtype=torch.float16, device=dev) for _ in range(n)]
 
-    # what ops.grouped_matmul does: one expert with few rows and a long k goes to the dense split-k entry point
-    ws_bytes = L.lib.aops_matmul_nt_workspace(rows, K, N) if E == 1 else 0
+    # what ops.grouped_matmul does: the two-phase entry (one expert with few rows and a long k wants scratch)
+    ws_bytes = L.lib.aops_grouped_matmul_workspace(rows, K, E, N)
     scratch = [torch.empty(ws_bytes, dtype=torch.uint8, device=dev) for _ in range(n)] if ws_bytes else None
 
     def mk(i):
-        if ws_bytes:
-            return lambda: L.check(L.lib.aops_matmul_nt_ws_f16(xs[i].data_ptr(), ws[i].data_ptr(), ys[i].data_ptr(),
-                                                               scratch[i].data_ptr(), ws_bytes, rows, K, N, L.stream()))
-        return lambda: L.check(L.lib.aops_grouped_matmul_f16(xs[i].data_ptr(), ws[i].data_ptr(), gd.data_ptr(),
-                                                            ys[i].data_ptr(), rows, K, E, N, L.stream()))
+        return lambda: L.check(L.lib.aops_grouped_matmul_ws_f16(
+            xs[i].data_ptr(), ws[i].data_ptr(), gd.data_ptr(), ys[i].data_ptr(),
+            scratch[i].data_ptr() if ws_bytes else None, ws_bytes, rows, K, E, N, L.stream()))
 
     med, mn = time_graph([mk(i) for i in range(n)], min_launches=40)
     if ws_bytes:
@@ -316,9 +342,7 @@ def _gmm_entry(L, ops, R, dev, cpu, op, config, x, w_storage, gl, note=None, che
     w_logical = w_storage.transpose(1, 2)
     cpu_ms = None
     if cpu:
-        t0 = time.perf_counter()
-        ref = R.grouped_matmul_ref(x, w_logical, gl)
-        cpu_ms = (time.perf_counter() - t0) * 1e3
+        cpu_ms, ref = time_cpu(lambda: R.grouped_matmul_ref(x, w_logical, gl))
         torch.testing.assert_close(ys[-1].cpu()[:end].float(), ref[:end].float(), rtol=2e-2, atol=2e-2)
     else:
         # check a slice of rows only (first experts) to keep the run short
@@ -514,7 +538,7 @@ def bench_moe(L, ops, R, dev, cpu):
     med, mn = time_graph([(lambda i=i: L.check(L.lib.aops_swiglu_f16(hs[i].data_ptr(), ys[i].data_ptr(), T, d, L.stream())))
                           for i in range(n)])
     h_cpu = h_dev.cpu()
-    cpu_ms = time_cpu(lambda: R.swiglu_ref(h_cpu)) if cpu else None
+    cpu_ms = time_cpu(lambda: R.swiglu_ref(h_cpu))[0] if cpu else None
     torch.testing.assert_close(ys[-1].cpu().float(), R.swiglu_ref(h_cpu).float(), rtol=1e-2, atol=1e-2)
     out.append(entry("swiglu", "4: MoE activation", f"x [{T},{2 * d}] f16", "hbm", alg, 0, med, mn, None, cpu_ms,
                      torch.get_num_threads()))
@@ -552,7 +576,7 @@ def bench_mlp(L, ops, R, dev, cpu):
     e1, h_dev = _gmm_entry(L, ops, R, dev, cpu, "grouped_matmul (E=1)", "3: MLP gate_up GEMM", x, gu[None], gl,
                            note="dense GEMM run as one expert; weight-stream bound, reported not scored")
     out.append(e1)
-    out.append(bench_swiglu(L, ops, R, dev, cpu, bs, inter, "3: MLP swiglu"))
+    out.append(bench_swiglu(L, ops, R, dev, cpu, bs, inter, "3: MLP swiglu", floor=True))
     h = ops.swiglu(h_dev)
     e2, y_dev = _gmm_entry(L, ops, R, dev, cpu, "grouped_matmul (E=1)", "3: MLP down GEMM", h.cpu(), dn[None], gl,
                            note="dense GEMM run as one expert; weight-stream bound, reported not scored")
@@ -650,13 +674,11 @@ def bench_paged_attention(L, ops, R, dev, cpu, wl):
     cpu_ms = None
     ref = None
     if cpu:
-        t0 = time.perf_counter()
-        ref = R.paged_attention_ref(wl.q, wl.kc, wl.vc, wl.bt, wl.ctx)
-        cpu_ms = (time.perf_counter() - t0) * 1e3
+        cpu_ms, ref = time_cpu(lambda: R.paged_attention_ref(wl.q, wl.kc, wl.vc, wl.bt, wl.ctx))
         torch.testing.assert_close(outs[0].cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
     e = entry("paged_attention", "5: decode attention", f"q [{B},{Hq},{D}], caches [{wl.NB},{Hkv * D // 16},{P},16], "
               f"sum(context)={wl.sum_ctx}", "hbm", wl.alg_bytes, 4 * wl.sum_ctx * Hq * D, med, mn, eager, cpu_ms,
-              torch.get_num_threads(), note="two kernels per call: split-KV partial + merge")
+              torch.get_num_threads(), note="one kernel per call: whole sequences per workgroup, longest first, no merge")
     e.pop("TFLOPs", None)
     e.pop("mfma_frac", None)
     # whole decode step: rope -> cache write -> attention (graph of the three C-ABI calls via the API)
@@ -666,6 +688,130 @@ def bench_paged_attention(L, ops, R, dev, cpu, wl):
     e["pipeline_fused_rope_cache_then_attention_api_eager_us"] = round(pipe2, 2)
     torch.testing.assert_close(wl.pipeline_fused(ops, 0).float(), wl.pipeline(ops, 0).float(), rtol=0, atol=0)
     return e
+
+
+
+def bench_pa_shape(L, R, dev, cpu, config, lens, Hq, Hkv, D, P, max_pages, note):
+    """Paged attention on another batch shape through the C ABI: graph-timed, oracle-checked.  These lines cover
+    the kernels the headline batch does not run: the balanced partition (pa_decode_balanced), its planning kernel
+    for more than 64 sequences (pa_plan_kernel), the merge (pa_decode_merge) and the generic kernel."""
+    import torch
+
+    B = len(lens)
+    g = torch.Generator().manual_seed(B + max_pages)
+    pages_per = [(l + P - 1) // P for l in lens]
+    NB = sum(pages_per) + 8
+    perm = torch.randperm(NB, generator=g)
+    bt = torch.zeros(B, max_pages, dtype=torch.int32)
+    c = 0
+    for b, npg in enumerate(pages_per):
+        bt[b, :npg] = perm[c:c + npg].int()
+        c += npg
+    cl = torch.tensor(lens, dtype=torch.int32)
+    q = torch.randn(B, Hq, D, generator=g).half()
+    kc = torch.empty(NB, Hkv * D // 16, P, 16, dtype=torch.float16)
+    vc = torch.empty_like(kc)
+    for i in range(0, NB, 64):
+        kc[i:i + 64] = torch.randn(min(64, NB - i), Hkv * D // 16, P, 16, generator=g).half()
+        vc[i:i + 64] = torch.randn(min(64, NB - i), Hkv * D // 16, P, 16, generator=g).half()
+    sum_ctx = int(sum(lens))
+    alg = sum_ctx * Hkv * D * 2 * 2 + 2 * B * Hq * D * 2 + bt.numel() * 4 + B * 4
+    cache_bytes = 2 * kc.numel() * 2
+    n = n_sets_for(cache_bytes, lo=2, hi=8)
+    qd, btd, cld = q.to(dev), bt.to(dev), cl.to(dev)
+    kcs = [kc.to(dev) for _ in range(n)]
+    vcs = [vc.to(dev) for _ in range(n)]
+    ws_bytes = L.lib.aops_paged_attention_workspace(B, Hq, Hkv, D, P, max_pages)
+    wss = [torch.empty(ws_bytes, dtype=torch.uint8, device=dev) for _ in range(n)]
+    outs = [torch.empty(B, Hq, D, dtype=torch.float16, device=dev) for _ in range(n)]
+
+    def mk(i):
+        return lambda: L.check(L.lib.aops_paged_attention_f16(
+            qd.data_ptr(), kcs[i].data_ptr(), vcs[i].data_ptr(), btd.data_ptr(), cld.data_ptr(), outs[i].data_ptr(),
+            wss[i].data_ptr(), ws_bytes, B, Hq, Hkv, D, P, max_pages, NB, L.stream()))
+
+    med, mn = time_graph([mk(i) for i in range(n)], min_launches=64)
+    cpu_ms = None
+    if cpu:
+        cpu_ms, ref = time_cpu(lambda: R.paged_attention_ref(q, kc, vc, bt, cl))
+    else:
+        ref = R.paged_attention_ref(q, kc, vc, bt, cl)
+    torch.testing.assert_close(outs[-1].cpu().float(), ref.float(), rtol=1e-2, atol=1e-2)
+    e = entry("paged_attention", config, f"q [{B},{Hq},{D}], block {P}, table width {max_pages} pages, sum(context)={sum_ctx}",
+              "hbm", alg, 0, med, mn, None, cpu_ms, torch.get_num_threads(), note)
+    e["workspace_bytes"] = ws_bytes
+    return e
+
+
+def bench_pa_more(L, R, dev, cpu):
+    import torch
+
+    g = torch.Generator().manual_seed(11)
+    ragged8 = torch.randint(512, 4097, (8,), generator=g).tolist()
+    skew64 = [32768] + [128] * 63
+    skew128 = [32768] + [128] * 127
+    return [
+        bench_pa_shape(L, R, dev, cpu, "5 at batch 8: contexts ~U[512,4096]", ragged8, 32, 8, 128, 128, 32,
+                       "pa_decode_balanced (one equal share of the token stream per CU) + pa_decode_merge"),
+        bench_pa_shape(L, R, dev, cpu, "5 at batch 1: one context of 32768 tokens", [32768], 32, 8, 128, 128, 256,
+                       "pa_decode_balanced + pa_decode_merge"),
+        bench_pa_shape(L, R, dev, cpu, "5 skewed: 64 sequences, one of 32768 tokens and 63 of 128", skew64, 32, 8, 128, 128, 256,
+                       "pa_decode_balanced + pa_decode_merge (a block table that allows more than 4096 tokens)"),
+        bench_pa_shape(L, R, dev, cpu, "5 skewed: 128 sequences, one of 32768 tokens and 127 of 128", skew128, 32, 8, 128, 128, 256,
+                       "pa_plan_kernel + pa_decode_balanced + pa_decode_merge (more sequences than lanes)"),
+        bench_pa_shape(L, R, dev, cpu, "5 with head_dim 96 (generic kernel): 16 sequences of 2048 tokens", [2048] * 16, 16, 4, 96,
+                       16, 128, "pa_decode_generic: head sizes other than 64/128/256"),
+    ]
+
+
+def bench_dense(L, R, dev):
+    """A compute-bound dense product through aops_matmul_nt_f16: HBM is out of the picture (805 MB against 1.1
+    TFLOP), so the line isolates the k loop of the persistent kernel the MoE GEMMs run."""
+    import torch
+
+    m = k = n = 8192
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(m, k, generator=g)).half()
+    w = (torch.randn(n, k, generator=g) / k ** 0.5).half()
+    xd, wd = x.to(dev), w.to(dev)
+    y = torch.empty(m, n, dtype=torch.float16, device=dev)
+    call = lambda: L.check(L.lib.aops_matmul_nt_f16(xd.data_ptr(), wd.data_ptr(), y.data_ptr(), m, k, n, L.stream()))
+    med, mn = time_graph([call], min_launches=32, trials=3)
+    rows = torch.randint(0, m, (48,), generator=g)
+    ref = x[rows].float() @ w.float().T
+    torch.testing.assert_close(y[rows.to(dev)].cpu().float(), ref, rtol=2e-2, atol=2e-2)
+    flops = 2 * m * k * n
+    alg = (m * k + n * k + m * n) * 2
+    e = entry("matmul", "dense 8192 x 8192 x 8192 (compute bound; not a BASELINE config)", f"x [{m},{k}] @ w [{n},{k}]^T f16",
+              "mfma", alg, flops, med, mn, None, None, 1,
+              "the persistent 320 x 256 kernel on one group; checked against the fp32 product on 48 sampled rows")
+    return e
+
+
+def kernel_source_digest():
+    """Digest of the paged-attention kernels' source: the recorded HBM-traffic figure names the digest it was
+    measured on and is dropped when the source has changed since."""
+    h = hashlib.sha256()
+    for name in ("paged_attention.hip", "aops_common.h"):
+        with open(os.path.join(ROOT, "ascend-ops_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def compact(e):
+    """One per_kernel record of the headline: operator, config, time, fraction of the bounding peak, CPU ms."""
+    if "error" in e:
+        return {"op": e.get("op_group"), "error": e["error"][:80]}
+    frac = e.get("mfma_frac") if e.get("bound") == "mfma" else e.get("hbm_frac")
+    c = {"op": e["op"], "config": e["config"].split(":")[0][:24], "us": round(e["gpu_us"], 1), "bound": e.get("bound"),
+         "frac": frac}
+    if "TFLOPs" in e and e.get("bound") == "mfma":
+        c["TFLOPs"] = e["TFLOPs"]
+    if "launch_floor_us" in e:
+        c["floor_us"] = e["launch_floor_us"]
+    if "cpu_ms" in e:
+        c["cpu_ms"] = round(e["cpu_ms"], 1)
+    return c
 
 
 # --------------------------------------------------------------------------------------- main
@@ -741,11 +887,13 @@ def main():
     del wl
     torch.cuda.empty_cache()
 
-    run("norm", lambda: bench_add_rms_norm(L, ops, R, dev, cpu, 128, "1: add_rms_norm"))
-    run("cache", lambda: bench_reshape_and_cache(L, ops, R, dev, cpu, 2048, "2: reshape_and_cache"))
-    run("rope", lambda: bench_rope(L, ops, R, dev, cpu, 64, "5: rope"))
+    run("norm", lambda: bench_add_rms_norm(L, ops, R, dev, cpu, 128, "1: add_rms_norm", floor=True))
+    run("cache", lambda: bench_reshape_and_cache(L, ops, R, dev, cpu, 2048, "2: reshape_and_cache", floor=True))
+    run("rope", lambda: bench_rope(L, ops, R, dev, cpu, 64, "5: rope", floor=True))
     run("mlp", lambda: bench_mlp(L, ops, R, dev, cpu))
     run("moe", lambda: bench_moe(L, ops, R, dev, cpu))
+    run("pa_more", lambda: bench_pa_more(L, R, dev, cpu))
+    run("dense", lambda: bench_dense(L, R, dev))
     run("scaled", lambda: [
         bench_add_rms_norm(L, ops, R, dev, False, 16384, "1 scaled x128: add_rms_norm",
                            "scaled shape: shows the kernel's asymptotic bandwidth, not a BASELINE config"),
@@ -769,18 +917,37 @@ def main():
         log("[bench] calibration copy done: 3 launches, 536870912 B read + 536870912 B written each")
         del src, dst
 
-    # HBM bytes per launch measured with rocprofv3 counters (recorded summary; None if absent)
-    traffic = None
+    # HBM bytes per launch measured with rocprofv3 counters: a recorded summary that names the digest of the kernel
+    # source it was measured on; a figure measured on other source is dropped (null) rather than reported stale
+    traffic, traffic_note = None, None
     tfile = os.path.join(ROOT, "profiles", "pa_decode_config5_hbm_traffic.txt")
     if os.path.exists(tfile):
+        recorded, digest = None, None
         for ln in open(tfile):
             if ln.strip().startswith("traffic_bytes_per_launch:"):
-                traffic = int(ln.split(":")[1])
+                recorded = int(ln.split(":")[1])
+            if ln.strip().startswith("kernel_source_digest:"):
+                digest = ln.split(":")[1].strip()
+        if recorded is not None and digest == kernel_source_digest():
+            traffic = recorded
+            traffic_note = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size; recorded in "
+                            "profiles/pa_decode_config5_hbm_traffic.txt for this kernel source")
+        else:
+            traffic_note = "recorded figure was measured on other kernel source (digest mismatch): dropped"
+
+    # the full per-operator records on their own line, BEFORE the headline (which must be the last line)
+    print(json.dumps({"per_op": per_op}), flush=True)
+
+    wanted = ("1:", "2:", "3: MLP swiglu", "5: rope", "4: MoE gate_up", "4: MoE down", "4: MoE gate_up + down",
+              "4: MoE gate_up + activation, fused", "5 at batch 8", "5 at batch 1", "5 skewed: 64", "dense 8192")
+    per_kernel = [compact(e) for e in per_op if "error" in e or any(e.get("config", "").startswith(w) for w in wanted)]
+    gmm_sum = next((e for e in per_op if e.get("config", "").startswith("4: MoE gate_up + down")), None)
+    gmm_cpu = [e.get("cpu_ms") for e in per_op if e.get("config") in ("4: MoE gate_up", "4: MoE down")]
 
     gbps_wall = alg_bytes / (ms_per_step * 1e-3) / 1e9
     gbps_kernel = alg_bytes / (pa["gpu_us"] * 1e-6) / 1e9
     line = {
-        "metric": "paged-attention decode HBM GB/s (algorithmic bytes / step); other operators under per_op",
+        "metric": "GB/s & % HBM roofline (norm/cache/PA); GMM TFLOPS & % fp16 MFMA peak",
         "value": round(gbps_wall, 1),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -793,8 +960,8 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {
-            "workload": "BASELINE configs[4]: paged-attention decode, batch 64, 32 q heads / 8 kv heads, head_dim 128, "
-                        "block 128, context ~U[512,4096], shuffled int32 block tables",
+            "workload": "BASELINE configs[4]: paged-attention decode, B=64, 32q/8kv heads, D=128, block 128, ctx~U[512,4096]",
+            "value_is": "paged-attention algorithmic bytes / wall step through the Python API",
             "sum_context_tokens": sum_ctx,
             "algorithmic_bytes_per_step": alg_bytes,
         },
@@ -805,22 +972,27 @@ def main():
             "unit": "GB/s",
             "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4),
             "traffic": traffic,
-            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known size; "
-                              "recorded in profiles/pa_decode_config5_hbm_traffic.txt" if traffic else None,
-            "kernel": "pa_decode_partial (split-KV main kernel; the merge kernel runs only when a sequence is split)",
+            "traffic_note": traffic_note,
+            "kernel": "pa_decode_partial<128,4,true>",
             "us_per_call": pa["gpu_us"],
+            "gmm": None if not gmm_sum else {
+                "config": "BASELINE configs[3] gate_up + down", "bound": "mfma", "TFLOPs": gmm_sum["TFLOPs"],
+                "peak": MFMA_F16_PEAK_TFLOPS, "frac": gmm_sum["mfma_frac"], "us": gmm_sum["gpu_us"],
+                "cpu_ms": None if not all(gmm_cpu) or len(gmm_cpu) != 2 else round(sum(gmm_cpu), 1),
+            },
+            "per_kernel": per_kernel,
         },
         "cpu_baseline": None if not cpu else {
             "value": round(alg_bytes / (pa["cpu_ms"] * 1e-3) / 1e9, 3),
             "unit": "GB/s",
             "cores": cores,
             "kind": "port",
-            "sample": "the full configs[4] batch (64 sequences), one pass of the torch fp32 oracle",
+            "sample": "the full configs[4] batch (64 sequences); torch fp32 oracle",
+            "runs": f"1 warm-up + median of {CPU_RUNS}",
             "ms": pa["cpu_ms"],
         },
-        "per_op": per_op,
     }
-    print(json.dumps(line), flush=True)
+    print(json.dumps(line, separators=(",", ":")), flush=True)
 
 
 if __name__ == "__main__":
