@@ -51,6 +51,8 @@ extern "C" const char* aops_strerror(int code) {
       return "workspace missing or too small";
     case AOPS_ERR_LAUNCH:
       return "HIP kernel launch failed";
+    case AOPS_ERR_SCRATCH_LIMIT:
+      return "problem needs more scratch than the fixed maximum of the entry point that allocates nothing";
     default:
       return "unknown error code";
   }

@@ -30,6 +30,8 @@
 // Semantics: signature, cache indexing, GQA mapping and the fixed 1/sqrt(D) scale follow
 // reference csrc/ffi/ops.cpp:408-482, csrc/opdev/op_host/paged_attention_ex.cpp:18-36 and
 // csrc/opdev/op_kernel/paged_attention_ex.cpp:90-99 (whose compute body is unfinished).
+#include <mutex>
+
 #include "aops_common.h"
 
 namespace aops {
@@ -902,6 +904,34 @@ static int pa_run(const void* q, const void* key_cache, const void* value_cache,
   return record_launch_status(hipGetLastError());
 }
 
+// Scratch of the entry point that allocates nothing: the partial results and the int area of the
+// split-KV kernels live in this array of the library's device image instead of a caller's workspace.
+// Every GPU the library runs on holds its own copy at its own address until the process ends.
+static __device__ __align__(256) unsigned char pa_static_scratch[AOPS_PA_NOALLOC_SCRATCH_BYTES];
+
+constexpr int kPaMaxDevices = 64;
+static std::mutex pa_scratch_mutex;
+static void* pa_scratch_addr[kPaMaxDevices];  // device address of pa_static_scratch per device, null = not looked up
+
+// Address of the current device's copy of the array.  In host code the array's name is only a handle
+// for hipGetSymbolAddress, never a device address.
+static int pa_scratch_for_current_device(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return record_launch_status(e);
+  if (dev < 0 || dev >= kPaMaxDevices) return AOPS_ERR_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> lock(pa_scratch_mutex);
+  if (!pa_scratch_addr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(pa_static_scratch));
+    if (e != hipSuccess) return record_launch_status(e);
+    if (!p) return AOPS_ERR_LAUNCH;
+    pa_scratch_addr[dev] = p;
+  }
+  *out = pa_scratch_addr[dev];
+  return AOPS_OK;
+}
+
 }  // namespace aops
 
 extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
@@ -914,4 +944,32 @@ extern "C" int aops_paged_attention_f16(const void* q, const void* key_cache,
   return aops::pa_run(q, key_cache, value_cache, block_tables, context_lens, o, workspace,
                       workspace_bytes, bs, num_heads, num_kv_heads, head_dim, block_size,
                       max_blocks_per_seq, num_blocks, stream);
+}
+
+extern "C" int aops_paged_attention_noalloc_f16(const void* q, const void* key_cache,
+                                                const void* value_cache,
+                                                const int32_t* block_tables,
+                                                const int32_t* context_lens, void* o, int64_t bs,
+                                                int64_t num_heads, int64_t num_kv_heads,
+                                                int64_t head_dim, int64_t block_size,
+                                                int64_t max_blocks_per_seq, int64_t num_blocks,
+                                                void* stream) {
+  using namespace aops;
+  if (!pa_args_valid(bs, num_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq))
+    return AOPS_ERR_INVALID_ARGUMENT;
+  // the size test comes first: a problem beyond the fixed maximum is refused whatever else is wrong
+  if (aops_paged_attention_workspace(bs, num_heads, num_kv_heads, head_dim, block_size,
+                                     max_blocks_per_seq) > (size_t)AOPS_PA_NOALLOC_SCRATCH_BYTES)
+    return AOPS_ERR_SCRATCH_LIMIT;
+  if (bs == 0) return AOPS_OK;
+  if (!q || !key_cache || !value_cache || !block_tables || !context_lens || !o)
+    return AOPS_ERR_INVALID_ARGUMENT;
+  void* scratch = nullptr;
+  const int rc = pa_scratch_for_current_device(&scratch);
+  if (rc != AOPS_OK) return rc;
+  // Nothing in the scratch has to start at zero: every partial result, plan entry and rank the
+  // kernels read in a call was written by an earlier kernel of the same call.
+  return pa_run(q, key_cache, value_cache, block_tables, context_lens, o, scratch,
+                (size_t)AOPS_PA_NOALLOC_SCRATCH_BYTES, bs, num_heads, num_kv_heads, head_dim,
+                block_size, max_blocks_per_seq, num_blocks, stream);
 }

@@ -31,6 +31,7 @@ extern "C" {
 #define AOPS_ERR_INVALID_ARGUMENT (-1) /* null pointer, negative size, size the kernels do not support */
 #define AOPS_ERR_WORKSPACE (-2)        /* workspace missing or too small */
 #define AOPS_ERR_LAUNCH (-3)           /* HIP reported an error at launch; see aops_last_hip_error() */
+#define AOPS_ERR_SCRATCH_LIMIT (-4)    /* aops_paged_attention_noalloc_f16: problem beyond its fixed scratch */
 
 /* Library version (major*10000 + minor*100 + patch). */
 int aops_version(void);
@@ -285,6 +286,30 @@ int aops_paged_attention_f16(const void* q, const void* key_cache, const void* v
                              int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
                              int64_t block_size, int64_t max_blocks_per_seq, int64_t num_blocks,
                              void* stream);
+
+/*
+ * aops_paged_attention_f16 for callers that cannot allocate device memory or pass a workspace (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference, whose binding allocates a workspace tensor per call
+ * (reference csrc/ffi/ops.cpp:454-461).  Same arguments, kernels and results as
+ * aops_paged_attention_f16, bit for bit, minus the workspace: the partial results of the split-KV
+ * kernels live in a fixed array of AOPS_PA_NOALLOC_SCRATCH_BYTES inside the library's device image
+ * (every GPU the library runs on holds its own copy until the process ends).  The call allocates
+ * and frees nothing.  The first call on a device looks up that device's address of the array
+ * (hipGetSymbolAddress, once per device); make it outside a graph capture.
+ * A problem whose aops_paged_attention_workspace() exceeds AOPS_PA_NOALLOC_SCRATCH_BYTES returns
+ * AOPS_ERR_SCRATCH_LIMIT and launches nothing.  All calls on one GPU share the one array, which keeps
+ * the previous call's contents (nothing in it needs clearing: every value a call reads it has written
+ * itself): calls that overlap on one GPU, on different streams or from different threads, race;
+ * calls on one stream are ordered and safe.
+ */
+#define AOPS_PA_NOALLOC_SCRATCH_BYTES (32 * 1024 * 1024)
+
+int aops_paged_attention_noalloc_f16(const void* q, const void* key_cache, const void* value_cache,
+                                     const int32_t* block_tables, const int32_t* context_lens,
+                                     void* o, int64_t bs, int64_t num_heads, int64_t num_kv_heads,
+                                     int64_t head_dim, int64_t block_size,
+                                     int64_t max_blocks_per_seq, int64_t num_blocks, void* stream);
 
 /*
  * Measurement aid: launches a kernel that does nothing, `workgroups` workgroups of `threads` threads

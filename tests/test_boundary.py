@@ -23,7 +23,7 @@ def test_library_loads_and_exports_every_declared_symbol():
     import ascend910a_extras
 
     declared = _declared_symbols()
-    assert len(declared) >= 25
+    assert len(declared) >= 26
     assert ascend910a_extras.LIBRARY_PATH == cabi.LIBRARY
     lib = ctypes.CDLL(ascend910a_extras.LIBRARY_PATH)
     for name in declared:
@@ -33,6 +33,7 @@ def test_library_loads_and_exports_every_declared_symbol():
     assert cabi.lib().aops_version() >= 200
     assert cabi.lib().aops_strerror(0) == b"success"
     assert b"workspace" in cabi.lib().aops_strerror(-2)
+    assert b"scratch" in cabi.lib().aops_strerror(-4)
 
 
 def test_extension_module_mirrors_the_reference_binding():
@@ -111,6 +112,11 @@ def test_c_abi_rejects_bad_sizes_without_touching_the_gpu():
     assert lib.aops_grouped_matmul_workspace(256, 14336, 2, 4096) == 0                                # only one expert is split over k
     assert lib.aops_grouped_matmul_ws_f16(None, None, None, None, None, 0, 16, 100, 2, 64, None) == -1
     assert lib.aops_grouped_matmul_ws_f16(None, None, None, None, None, 0, 0, 64, 2, 64, None) == 0
+    # the entry point that allocates nothing: argument and size checks come before any device work
+    assert lib.aops_paged_attention_noalloc_f16(None, None, None, None, None, None, 2, 8, 2, 72, 128, 4, 16, None) == -1
+    assert lib.aops_paged_attention_noalloc_f16(None, None, None, None, None, None, 0, 8, 2, 128, 128, 4, 16, None) == 0
+    assert lib.aops_paged_attention_workspace(4096, 32, 8, 128, 128, 256) > 32 * 1024 * 1024
+    assert lib.aops_paged_attention_noalloc_f16(None, None, None, None, None, None, 4096, 32, 8, 128, 128, 256, 16, None) == -4
     # fused extensions
     assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 160, 2, 128, None) == -1   # k % 64
     assert lib.aops_grouped_matmul_swiglu_f16(None, None, None, None, 16, 128, 2, 96, None) == -1    # n % 64
