@@ -10,6 +10,7 @@
 // Host code only (no kernels): compiled with the C++ compiler against the torch headers and linked
 // against libaops.so, which sits next to the module.
 #include <ATen/ATen.h>
+#include <ATen/hip/EmptyTensor.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <c10/hip/HIPStream.h>
 #include <pybind11/pybind11.h>
@@ -86,9 +87,14 @@ void status(const char* op, int code) {
   TORCH_CHECK(false, op, ": ", aops_strerror(code));
 }
 
-Tensor scratch(const Tensor& like, size_t bytes) {
-  return at::empty({(int64_t)bytes}, like.options().dtype(at::kByte));
+// Output allocation straight from the caching allocator (what at::empty arrives at after its dispatch):
+// the operators of a decode step take a few microseconds, so the host cost per call matters.
+Tensor fresh(const Tensor& like, at::IntArrayRef sizes, at::ScalarType dtype) {
+  return Tensor(at::detail::empty_cuda(sizes, dtype, like.device(), std::nullopt));
 }
+Tensor fresh_like(const Tensor& t) { return fresh(t, t.sizes(), t.scalar_type()); }
+
+Tensor scratch(const Tensor& like, size_t bytes) { return fresh(like, {(int64_t)bytes}, at::kByte); }
 
 // ---- the reference's six operators ---------------------------------------------------------------
 
@@ -116,8 +122,8 @@ std::vector<Tensor> rope(const Tensor& q, const Tensor& k, const Tensor& positio
                           {"position_ids", position_ids, at::kInt},
                           {"cos_cache", cos_cache, at::kHalf},
                           {"sin_cache", sin_cache, at::kHalf}});
-  Tensor out_q = at::empty_like(q);
-  Tensor out_k = at::empty_like(k);
+  Tensor out_q = fresh_like(q);
+  Tensor out_k = fresh_like(k);
   Launch l(q);
   status("rope", aops_rope_neox_f16(dev_ptr(q), dev_ptr(k), static_cast<const int32_t*>(dev_ptr(position_ids)),
                                     dev_ptr(cos_cache), dev_ptr(sin_cache), dev_ptr(out_q), dev_ptr(out_k), bs,
@@ -132,7 +138,7 @@ Tensor swiglu(const Tensor& x) {
               x.size(-1));
   TORCH_CHECK(x.is_contiguous(), "swiglu: input tensor must be contiguous");
   require_device("swiglu", {{"x", x, at::kHalf}});
-  Tensor y = at::empty({x.size(0), x.size(1) / 2}, x.options());
+  Tensor y = fresh(x, {x.size(0), x.size(1) / 2}, x.scalar_type());
   Launch l(x);
   status("swiglu", aops_swiglu_f16(dev_ptr(x), dev_ptr(y), x.size(0), x.size(1) / 2, l.stream));
   return y;
@@ -162,7 +168,7 @@ void check_grouped_matmul(const char* name, const Tensor& x, const Tensor& w, co
 Tensor grouped_matmul(const Tensor& x, const Tensor& w, const Tensor& group_list) {
   check_grouped_matmul("grouped_matmul", x, w, group_list);
   const int64_t rows = x.size(0), dim = x.size(1), num_experts = w.size(0), inner_dim = w.size(2);
-  Tensor y = at::empty({rows, inner_dim}, x.options());
+  Tensor y = fresh(x, {rows, inner_dim}, x.scalar_type());
   Launch l(x);
   const size_t ws_bytes = aops_grouped_matmul_workspace(rows, dim, num_experts, inner_dim);
   Tensor ws;
@@ -189,8 +195,8 @@ std::tuple<Tensor, Tensor> add_rms_norm(const Tensor& x, const Tensor& residual,
   TORCH_CHECK(x.size(1) % 64 == 0, "add_rms_norm: last dimension must be a multiple of 64, got ", x.size(1));
   require_device("add_rms_norm",
                  {{"x", x, at::kHalf}, {"residual", residual, at::kHalf}, {"weight", weight, at::kHalf}});
-  Tensor y = at::empty_like(x);
-  Tensor residual_output = at::empty_like(x);
+  Tensor y = fresh_like(x);
+  Tensor residual_output = fresh_like(x);
   Launch l(x);
   status("add_rms_norm",
          aops_add_rms_norm_f16(dev_ptr(x), dev_ptr(residual), dev_ptr(weight), (float)epsilon, dev_ptr(y),
@@ -271,7 +277,7 @@ Tensor paged_attention(const Tensor& q, const Tensor& key_cache, const Tensor& v
                                      {"block_tables", block_tables, at::kInt},
                                      {"context_lens", context_lens, at::kInt}});
   const int64_t max_blocks = block_tables.size(1);
-  Tensor o = at::empty_like(q);
+  Tensor o = fresh_like(q);
   if (bs == 0) return o;
   Launch l(q);
   const size_t ws_bytes =
@@ -307,7 +313,7 @@ Tensor matmul(const Tensor& x, const Tensor& w) {
   const int64_t m = x.size(0), k = x.size(1), n = w.size(0);
   TORCH_CHECK(k % 64 == 0 && n % 64 == 0, "matmul: k and n must be multiples of 64, got k=", k, " and n=", n);
   require_device("matmul", {{"x", x, at::kHalf}, {"w", w, at::kHalf}});
-  Tensor y = at::empty({m, n}, x.options());
+  Tensor y = fresh(x, {m, n}, x.scalar_type());
   Launch l(x);
   const size_t ws_bytes = m > 0 ? aops_matmul_nt_workspace(m, k, n) : 0;
   Tensor ws;
@@ -322,7 +328,7 @@ Tensor matmul(const Tensor& x, const Tensor& w) {
 Tensor grouped_matmul_swiglu(const Tensor& x, const Tensor& w, const Tensor& group_list) {
   check_grouped_matmul("grouped_matmul_swiglu", x, w, group_list);
   const int64_t rows = x.size(0), dim = x.size(1), num_experts = w.size(0), inner_dim = w.size(2);
-  Tensor y = at::empty({rows, inner_dim / 2}, x.options());
+  Tensor y = fresh(x, {rows, inner_dim / 2}, x.scalar_type());
   Launch l(x);
   status("grouped_matmul_swiglu",
          aops_grouped_matmul_swiglu_f16(dev_ptr(x), dev_ptr(w), static_cast<const int64_t*>(dev_ptr(group_list)),
@@ -342,7 +348,7 @@ Tensor moe_gather(const Tensor& x, const Tensor& sorted_idx, const Tensor& group
   require_device("moe_gather",
                  {{"x", x, at::kHalf}, {"sorted_idx", sorted_idx, at::kInt}, {"group_list", group_list, at::kLong}});
   const int64_t n = sorted_idx.numel();
-  Tensor out = at::empty({n, x.size(1)}, x.options());
+  Tensor out = fresh(x, {n, x.size(1)}, x.scalar_type());
   Launch l(x);
   status("moe_gather",
          aops_moe_gather_f16(dev_ptr(x), static_cast<const int32_t*>(dev_ptr(sorted_idx)),
@@ -377,7 +383,7 @@ Tensor grouped_matmul_swiglu_gather(const Tensor& x, const Tensor& sorted_idx, i
                         {"w", w, at::kHalf},
                         {"group_list", group_list, at::kLong},
                         {"sorted_idx", sorted_idx, at::kInt}});
-  Tensor y = at::empty({rows, inner_dim / 2}, x.options());
+  Tensor y = fresh(x, {rows, inner_dim / 2}, x.scalar_type());
   Launch l(x);
   status(name, aops_grouped_matmul_swiglu_gather_f16(
                    dev_ptr(x), static_cast<const int32_t*>(dev_ptr(sorted_idx)), topk, x.size(0), dev_ptr(w),
@@ -424,9 +430,9 @@ py::object rope_reshape_and_cache(const Tensor& q, const Tensor& k, const Tensor
                         {"key_cache", key_cache, at::kHalf},
                         {"value_cache", value_cache, at::kHalf},
                         {"slot_indices", slot_indices, at::kInt}});
-  Tensor out_q = at::empty_like(q);
+  Tensor out_q = fresh_like(q);
   Tensor out_k;
-  if (return_k) out_k = at::empty_like(k);
+  if (return_k) out_k = fresh_like(k);
   Launch l(q);
   int code;
   if (norm) {
@@ -461,9 +467,9 @@ std::tuple<Tensor, Tensor, Tensor> moe_sort(const Tensor& topk_ids, int64_t num_
   TORCH_CHECK(num_experts > 0 && num_experts <= 4095, "moe_sort: num_experts must be in 1..4095, got ", num_experts);
   require_device("moe_sort", {{"topk_ids", topk_ids, at::kInt}});
   const int64_t n = topk_ids.numel();
-  Tensor sorted_idx = at::empty({n}, topk_ids.options());
-  Tensor inverse_idx = at::empty({n}, topk_ids.options());
-  Tensor group_list = at::empty({num_experts}, topk_ids.options().dtype(at::kLong));
+  Tensor sorted_idx = fresh(topk_ids, {n}, topk_ids.scalar_type());
+  Tensor inverse_idx = fresh(topk_ids, {n}, topk_ids.scalar_type());
+  Tensor group_list = fresh(topk_ids, {num_experts}, at::kLong);
   Launch l(topk_ids);
   const size_t ws_bytes = aops_moe_sort_workspace(n, num_experts);
   TORCH_CHECK(ws_bytes > 0, "moe_sort: unsupported size n=", n, ", num_experts=", num_experts);
@@ -490,7 +496,7 @@ Tensor moe_combine(const Tensor& y, const Tensor& inverse_idx, const Tensor& top
                                  {"inverse_idx", inverse_idx, at::kInt},
                                  {"topk_weights", topk_weights, at::kFloat},
                                  {"topk_ids", topk_ids, at::kInt}});
-  Tensor out = at::empty({tokens, y.size(1)}, y.options());
+  Tensor out = fresh(y, {tokens, y.size(1)}, y.scalar_type());
   Launch l(y);
   status("moe_combine",
          aops_moe_combine_f16(dev_ptr(y), static_cast<const int32_t*>(dev_ptr(inverse_idx)),

@@ -223,20 +223,21 @@ __device__ __forceinline__ GmmPlan gmm_make_plan(const int64_t* __restrict__ gro
 // Work item `work` (0 <= work < total_tiles * n_tiles) -> (expert, m-tile, n-tile); the m-tiles
 // that share a weight tile are adjacent.  With at most kBndCache experts per lane nothing is
 // read from memory.
-template <int kBM>
+// Index: int64_t, or int where the launcher has checked that the number of work items fits (the
+// persistent kernel: 32-bit uniform values stay in scalar registers); `lane`: the caller's lane id.
+template <int kBM, typename Index>
 __device__ __forceinline__ GmmWork gmm_locate(const GmmPlan& p,
                                               const int64_t* __restrict__ group_list,
                                               int num_experts, int64_t rows, int n_tiles,
-                                              int64_t work) {
-  const int lane = threadIdx.x & (kWave - 1);
+                                              Index work, int lane) {
   auto clampr = [&](int64_t v) -> int { return (int)(v < 0 ? 0 : (v > rows ? rows : v)); };
-  const int64_t lo = (int64_t)(p.incl - p.tiles) * n_tiles;
-  const int64_t hi = (int64_t)p.incl * n_tiles;
+  const Index lo = (Index)(p.incl - p.tiles) * n_tiles;
+  const Index hi = (Index)p.incl * n_tiles;
   const bool mine = work >= lo && work < hi;
   int f_expert = 0, f_begin = 0, f_end = 0, f_ntile = 0;
   if (mine) {
     const int e0 = lane * p.per;
-    int64_t base = lo;
+    Index base = lo;
     if (p.per <= kBndCache) {
       int prev = p.bnd[0];
       bool found = false;
@@ -244,7 +245,7 @@ __device__ __forceinline__ GmmWork gmm_locate(const GmmPlan& p,
       for (int j = 0; j < kBndCache; ++j) {
         const int end = p.bnd[j + 1];
         const int t = (j < p.per && end > prev) ? (end - prev + kBM - 1) / kBM : 0;
-        const int64_t span = (int64_t)t * n_tiles;
+        const Index span = (Index)t * n_tiles;
         if (!found && t > 0 && work < base + span) {
           const int local = (int)(work - base);
           f_expert = e0 + j;
@@ -264,7 +265,7 @@ __device__ __forceinline__ GmmWork gmm_locate(const GmmPlan& p,
         if (e >= num_experts) break;
         const int end = clampr(gmm_group_end(group_list, e, rows));
         const int t = end > prev ? (end - prev + kBM - 1) / kBM : 0;
-        const int64_t span = (int64_t)t * n_tiles;
+        const Index span = (Index)t * n_tiles;
         if (work < base + span) {
           const int local = (int)(work - base);
           f_expert = e;

@@ -24,6 +24,20 @@ namespace aops {
 // row_idx[j] / idx_div of x (the routing order of a mixture of experts: row_idx = the sorted flat
 // routing indices, idx_div = top-k), so the expert-sorted copy of x never exists.  The tile's
 // source rows are looked up once per work item.
+// Lane id taken from the hardware each time, through a volatile asm the compiler neither hoists nor
+// merges.  The persistent kernel derives its per-item offsets from it instead of from values computed at
+// kernel start: those would have to live across the k loop, where the accumulators fill the register
+// file, and so be spilled - and reloading a spilled register means waiting for every outstanding memory
+// operation, the next item's operand copies and this item's stores included.
+__device__ __forceinline__ int lane_id_fresh() {
+  int l;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+  return l;
+}
+
+constexpr int kPlanInts = 2 + kBndCache + 1;  // per-lane record of the group_list scan kept in LDS
+constexpr int kEpiScratchHalfs = 512;         // 1 KiB of LDS per wave for the epilogue's row transposition
+
 template <int MB, int NB, int WN, bool SWIGLU, bool GATHER>
 __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kernel(
     const f16* __restrict__ x, const f16* __restrict__ w, const int64_t* __restrict__ group_list,
@@ -43,7 +57,8 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   extern __shared__ __attribute__((aligned(16))) f16 smem[];
   f16* sa = smem;                         // [2][BM * kBK]
   f16* sb = smem + 2 * BM * kBK;          // [2][BN * kBK]
-  int* splan = reinterpret_cast<int*>(smem + 2 * (BM + BN) * kBK);  // [kWaves][kWave][8]
+  int* splan = reinterpret_cast<int*>(smem + 2 * (BM + BN) * kBK);  // [kWave][kPlanInts], the same in every wave
+  f16* sepi = reinterpret_cast<f16*>(splan + kWave * kPlanInts);     // [kWaves][kEpiScratchHalfs]
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -53,7 +68,9 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   const int n_tiles = (n_out + BNO - 1) / BNO;
   const int ktiles = k / kBK;
 
-  int* my_plan = splan + (wave * kWave + lane) * 8;
+  // every wave computes the same scan and stores it to the same place: a wave reads back values that it
+  // (or another wave, identically) wrote, so no synchronisation is needed
+  int* my_plan = splan + lane * kPlanInts;
   int plan_per, plan_total;
   {
     const GmmPlan plan = gmm_make_plan<BM>(group_list, num_experts, rows);
@@ -64,30 +81,34 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
 #pragma unroll
     for (int j = 0; j <= kBndCache; ++j) my_plan[2 + j] = plan.bnd[j];
   }
-  const int64_t total_work = (int64_t)plan_total * n_tiles;
-  const int64_t share = (total_work + kXcds - 1) / kXcds;
+  // 32-bit on purpose (the launcher refuses problems with 2^31 work items or more): uniform 32-bit values
+  // stay in scalar registers, 64-bit ones ended up in vector registers and were spilled
+  const int total_work = __builtin_amdgcn_readfirstlane(plan_total * n_tiles);
+  const int share = (total_work + kXcds - 1) / kXcds;
   const int xcd = blockIdx.x % kXcds;
   const int wg_in_xcd = blockIdx.x / kXcds;
   const int wgs_per_xcd = gridDim.x / kXcds;
-  auto locate = [&](int64_t local) -> GmmWork {
-    const int64_t item = (int64_t)xcd * share + local;
+  auto locate = [&](int local) -> GmmWork {
+    const int item = xcd * share + local;
     if (local >= share || item >= total_work) {
       GmmWork none;
       none.valid = false;
       none.expert = none.row_begin = none.row_end = none.n_tile = 0;
       return none;
     }
-    GmmPlan plan;  // this lane's part, written by this lane: no synchronisation needed
+    GmmPlan plan;  // this lane's part, written by this lane (and identically by its twins in the other waves)
+    const int lane_l = lane_id_fresh();
+    const int* my_plan = splan + lane_l * kPlanInts;
     plan.per = plan_per;
     plan.total_tiles = plan_total;
     plan.tiles = my_plan[0];
     plan.incl = my_plan[1];
 #pragma unroll
     for (int j = 0; j <= kBndCache; ++j) plan.bnd[j] = my_plan[2 + j];
-    return gmm_locate<BM>(plan, group_list, num_experts, rows, n_tiles, item);
+    return gmm_locate<BM, int>(plan, group_list, num_experts, rows, n_tiles, item, lane_l);
   };
 
-  int64_t local = wg_in_xcd;
+  int local = wg_in_xcd;
   GmmWork cur = locate(local);
   if (!cur.valid) return;
 
@@ -110,6 +131,9 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   // number of valid 32-column blocks of the item instead of an offset.
   const uint32_t off0_glu = ((uint32_t)(lane_row & 31) + (lane_row >= 32 ? (uint32_t)n_out : 0u)) * (uint32_t)k + lane_c * 8;
   auto set_sources = [&](const GmmWork& it) {
+    const int lane_s = lane_id_fresh();
+    const int lane_row = wave * 8 + ((lane_s >> 3) ^ (wave & 1));
+    const int lane_c = (lane_s & 7) ^ (lane_row & 7);
     b_base = w + ((int64_t)it.expert * n + (int64_t)it.n_tile * BNO) * k;
     const int n_left = min(n_out - it.n_tile * BNO, BNO);
     const int x_left = min(it.row_end - it.row_begin, BM);  // rows of the group in this tile
@@ -270,77 +294,69 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     }
 
     // Epilogue of `cur`.  acc[i][j][4g+e]: output row 32*(wm+2i) + fm, output column
-    // wn*32*NB + 32j + 8g + 4fq + e.  For a pair of column groups (g, g+1) the two lanes of a row
-    // (fq = 0, 1) exchange halves: v_permlane32_swap trades the upper 32 lanes of its first
-    // operand for the lower 32 lanes of its second, after which lane fq holds the 8 consecutive
-    // columns of group g+fq.
-    const int m_w = 32 * wm + fm;
-    if constexpr (SWIGLU) {
-      const int col_w = cur.n_tile * BNO + wn * 32;
+    // wn*32*NB + 32j + 8g + 4fq + e: a lane holds one output row and, of the wave's columns, 8-byte
+    // pieces that alternate with those of its partner lane (fq).  Stored from there, every store
+    // instruction would scatter 32-byte pieces over 32 rows, and the count of write requests, not their
+    // bytes, is what the memory pipeline of a CU charges for.  So the rows go through a 1 KiB LDS scratch
+    // of the wave's own, a few at a time: the lanes of those rows write their pieces (16-byte slots
+    // XOR-swizzled by the row: no bank conflicts either way), then all 64 lanes read 16 bytes each in row
+    // order and store whole row segments - eight 128-byte lines per instruction (SWIGLU: sixteen 64-byte
+    // halves).  The operand stages stay untouched: the next item's first tiles are landing in them.
+    {
+      f16* scr = sepi + wave * kEpiScratchHalfs;
+      constexpr int kSegHalfs = SWIGLU ? 32 : 32 * NB;       // output columns of the wave
+      constexpr int kRowsPerUnit = kEpiScratchHalfs / kSegHalfs;  // 8 rows of 128 bytes, or 16 of 64
+      constexpr int kSlots = kSegHalfs / 8;                  // 16-byte slots per row segment
+      constexpr int kUnits = 32 / kRowsPerUnit;
+      static_assert(kSegHalfs == 64 || kSegHalfs == 32, "row segment of 128 or 64 bytes");
+      const int col_w = SWIGLU ? cur.n_tile * BNO + wn * 32 : cur.n_tile * BN + wn * 32 * NB;
+      // the lane-derived offsets are the same for every item; taken from a fresh lane id they are not
+      // hoisted out of the item loop (and spilled)
+      const int lane_e = lane_id_fresh();
+      const int fm_e = lane_e & 31;
+      const int fq_e = lane_e >> 5;
+      const int unit_of_lane = fm_e / kRowsPerUnit;
+      const int r_w = fm_e % kRowsPerUnit;                    // this lane's row inside its unit
+      const int r_r = lane_e / kSlots;                        // the row this lane reads back and stores
+      const int q_r = lane_e % kSlots;                        // ... and its 16-byte slot
+      // slot swizzle of row r: rows whose segments start in the same bank get different slot orders
+      auto swz = [](int r) { return kSlots == 8 ? (r & 7) : ((r ^ (r >> 2)) & 3); };
+      const f16* rd = scr + r_r * kSegHalfs + ((q_r ^ swz(r_r)) * 8);
 #pragma unroll
       for (int i = 0; i < MB; ++i) {
-        const int m = m_w + 64 * i;
         if (i < live && col_w < n_out) {  // wave uniform
-          const bool row_ok = m < tile_rows;
-          f16* yrow = y + (int64_t)(cur.row_begin + m) * n_out + col_w + 8 * fq;
+          // (the conversion sits inside the branch of the lane's unit: no registers are held for the pieces)
 #pragma unroll
-          for (int gp = 0; gp < 2; ++gp) {
-            f16x4 p0, p1;
+          for (int u = 0; u < kUnits; ++u) {
+            if (unit_of_lane == u) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-              const float g = acc[i][0][8 * gp + e];
-              const float u = acc[i][1][8 * gp + e];
-              const float ex = __builtin_amdgcn_exp2f(-1.4426950408889634f * g);
-              const f16 o = (f16)(g * u * __builtin_amdgcn_rcpf(1.0f + ex));
-              if (e < 4) p0[e] = o; else p1[e - 4] = o;
-            }
-            const u32x2 d0 = __builtin_bit_cast(u32x2, p0);
-            const u32x2 d1 = __builtin_bit_cast(u32x2, p1);
-            const auto lo = __builtin_amdgcn_permlane32_swap(d0[0], d1[0], false, false);
-            const auto hi = __builtin_amdgcn_permlane32_swap(d0[1], d1[1], false, false);
-            u32x4 out;
-            out[0] = lo[0];
-            out[1] = hi[0];
-            out[2] = lo[1];
-            out[3] = hi[1];
-            if (row_ok) st128(yrow + 16 * gp, __builtin_bit_cast(f16x8, out));
-          }
-        }
-      }
-    } else {
-    const int col_w = cur.n_tile * BN + wn * 32 * NB;
+              for (int q = 0; q < kSlots; ++q) {
+                f16x4 piece;  // slot q of this lane's row, its fq half
 #pragma unroll
-    for (int i = 0; i < MB; ++i) {
-      const int m = m_w + 64 * i;
-      if (i < live) {  // wave uniform: both lanes of every pair take part in the exchange
-        const bool row_ok = m < tile_rows;
-        f16* yrow = y + (int64_t)(cur.row_begin + m) * n + col_w + 8 * fq;
-#pragma unroll
-        for (int j = 0; j < NB; ++j) {
-          if (col_w + 32 * j < n) {
-#pragma unroll
-            for (int gp = 0; gp < 2; ++gp) {
-              f16x4 p0, p1;
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                p0[e] = (f16)acc[i][j][8 * gp + e];
-                p1[e] = (f16)acc[i][j][8 * gp + 4 + e];
+                for (int e = 0; e < 4; ++e) {
+                  if constexpr (SWIGLU) {
+                    const float gt = acc[i][0][4 * q + e];
+                    const float up = acc[i][1][4 * q + e];
+                    const float ex = __builtin_amdgcn_exp2f(-1.4426950408889634f * gt);
+                    piece[e] = (f16)(gt * up * __builtin_amdgcn_rcpf(1.0f + ex));
+                  } else {
+                    piece[e] = (f16)acc[i][q / 4][4 * (q % 4) + e];
+                  }
+                }
+                *reinterpret_cast<f16x4*>(scr + r_w * kSegHalfs + ((q ^ swz(r_w)) * 8) + 4 * fq_e) = piece;
               }
-              const u32x2 d0 = __builtin_bit_cast(u32x2, p0);
-              const u32x2 d1 = __builtin_bit_cast(u32x2, p1);
-              const auto lo = __builtin_amdgcn_permlane32_swap(d0[0], d1[0], false, false);
-              const auto hi = __builtin_amdgcn_permlane32_swap(d0[1], d1[1], false, false);
-              u32x4 out;
-              out[0] = lo[0];
-              out[1] = hi[0];
-              out[2] = lo[1];
-              out[3] = hi[1];
-              if (row_ok) st128(yrow + 32 * j + 16 * gp, __builtin_bit_cast(f16x8, out));
             }
+            // LDS serves a wave's accesses in order: the read sees the writes above, and the next unit's
+            // writes come after this read
+            asm volatile("" ::: "memory");
+            const f16x8 v = *reinterpret_cast<const f16x8*>(rd);
+            asm volatile("" ::: "memory");
+            const int m = 32 * wm + 64 * i + u * kRowsPerUnit + r_r;
+            if (m < tile_rows)
+              st128(y + (int64_t)(cur.row_begin + m) * n_out + col_w + q_r * 8, v);
           }
         }
       }
-    }
     }
     if (!nxt.valid) break;
     cur = nxt;
@@ -356,13 +372,15 @@ static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* grou
   constexpr int BM = 64 * MB;
   constexpr int BN = 32 * NB * WN;
   constexpr int kWaves = 2 * WN;
-  constexpr int kLds = 2 * (BM + BN) * kBK * (int)sizeof(f16) + kWaves * kWave * 8 * (int)sizeof(int);
+  constexpr int kLds = 2 * (BM + BN) * kBK * (int)sizeof(f16) + kWave * kPlanInts * (int)sizeof(int) +
+                       kWaves * kEpiScratchHalfs * (int)sizeof(f16);
   static_assert(kLds <= 160 * 1024, "LDS budget");
   const int cus = device_cu_count();
   constexpr int BNO = SWIGLU ? BN / 2 : BN;
   const int64_t n_out = SWIGLU ? n / 2 : n;
   const int64_t n_tiles = (n_out + BNO - 1) / BNO;
   const int64_t max_work = ((rows + BM - 1) / BM + num_experts) * n_tiles;
+  if (max_work > 0x7fffffff - 8 * kXcds) return AOPS_ERR_INVALID_ARGUMENT;  // the kernel counts work items in 32 bits
   int64_t grid = cus < max_work ? cus : max_work;
   grid = grid / kXcds * kXcds;
   if (grid < kXcds) grid = kXcds;

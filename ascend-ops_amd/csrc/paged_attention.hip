@@ -49,6 +49,7 @@ struct PaChunking {
 
 constexpr int kPaUnit = kPaWaves * kPaStep;  // 256 tokens: one step of every wave
 constexpr int kPaMaxGroup = 16;              // query heads per kv head the matrix-core kernel serves
+constexpr int kPaXcds = 8;                   // workgroup i runs on XCD i % 8
 
 // Batches of up to kPaPlanMax sequences can use the balanced partition; above 64 sequences it is
 // computed by a one-workgroup kernel into kPaPlanInts(bs) ints behind the partial results.
@@ -727,74 +728,122 @@ static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t*
 }
 
 // Generic path for every other shape (head_dim a multiple of 16 up to 256, any block size, any
-// whole number of query heads per kv head): one workgroup of four waves per (sequence, query
-// head); a wave takes every fourth token, its lanes split head_dim, scores are finished with a
-// wave reduction, every wave keeps its own running softmax and the four are merged through LDS.
-// Correct for all shapes the cache layout allows, not tuned: 2-byte loads.
+// whole number of query heads per kv head): one workgroup of four waves per (sequence, query head).
+// A wave takes every fourth block of 32 tokens; lane (token = lane / 2, half = lane % 2) loads, d-chunk
+// row by d-chunk row, the 16 bytes that hold d = 16c + 8*half ..+7 of its token, so that a load
+// instruction of a wave covers 1 KiB of consecutive tokens of one d-chunk row (tokens of one page are
+// adjacent in the layout).  Scores are finished with one exchange between the two lanes of a token, the
+// block's softmax with wave reductions; every lane accumulates p * V for its own token and half, and the
+// 32 tokens are added up with lane exchanges once per wave at the end.  The four waves meet in LDS.
+// Workgroups are renumbered so that the query heads of one kv head, which read the same K and V, run on
+// one XCD side by side and share its L2.  CH = number of d-chunk rows the registers are sized for.
 constexpr int kPaGenericMaxD = 256;
+constexpr int kPaGenericWaves = 4;
 
-__global__ __launch_bounds__(4 * kWave) void pa_decode_generic(
+template <int CH>
+__global__ __launch_bounds__(kPaGenericWaves* kWave) void pa_decode_generic(
     const f16* __restrict__ q, const f16* __restrict__ key_cache,
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
-    const int32_t* __restrict__ context_lens, f16* __restrict__ out, int num_heads,
+    const int32_t* __restrict__ context_lens, f16* __restrict__ out, int bs, int num_heads,
     int num_kv_heads, int head_dim, int block_size, int max_blocks_per_seq, float scale_log2,
     int num_blocks) {
-  constexpr int kPerLane = kPaGenericMaxD / kWave;
-  const int h = blockIdx.x;
-  const int b = blockIdx.y;
+  // XCD x takes the contiguous range [x * share, (x + 1) * share) of the (sequence, head) pairs
+  const int total = bs * num_heads;
+  const int share = (total + kPaXcds - 1) / kPaXcds;
+  const int item = (int)(blockIdx.x % kPaXcds) * share + (int)(blockIdx.x / kPaXcds);
+  if ((int)(blockIdx.x / kPaXcds) >= share || item >= total) return;
+  const int b = item / num_heads;
+  const int h = item - b * num_heads;
   const int g = h / (num_heads / num_kv_heads);
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int lane = threadIdx.x & (kWave - 1);
+  const int tok = lane >> 1;
+  const int half = lane & 1;
+  const int chunks = head_dim / 16;
   const int context_len = min(context_lens[b], max_blocks_per_seq * block_size);
-  const int64_t row_chunks = (int64_t)num_kv_heads * head_dim / 16;  // 32-byte granules per token
+  const int64_t row_chunks = (int64_t)num_kv_heads * chunks;  // 32-byte granules per token
   const int32_t* table = block_tables + (int64_t)b * max_blocks_per_seq;
 
-  float qf[kPerLane], acc[kPerLane];
-  int64_t elem_off[kPerLane];  // offset of (head g, dim d) inside a page, token 0
+  f16x8 qv[CH];
+  float acc[CH][8];
 #pragma unroll
-  for (int i = 0; i < kPerLane; ++i) {
-    const int d = lane + kWave * i;
-    const bool live = d < head_dim;
-    qf[i] = live ? (float)q[((int64_t)b * num_heads + h) * head_dim + d] : 0.f;
-    acc[i] = 0.f;
-    const int f = g * head_dim + (live ? d : 0);
-    elem_off[i] = (int64_t)(f / 16) * block_size * 16 + (f % 16);
+  for (int c = 0; c < CH; ++c) {
+    const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    qv[c] = c < chunks ? ld128(q + ((int64_t)b * num_heads + h) * head_dim + 16 * c + 8 * half) : zero8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[c][e] = 0.f;
   }
-  float m = kNegBig, l = 0.f;
-  for (int j = wave; j < context_len; j += 4) {
-    const int blk = j / block_size;
-    const int64_t base = (int64_t)min(max(table[blk], 0), num_blocks - 1) * row_chunks * block_size * 16 +
-                         (int64_t)(j - blk * block_size) * 16;
-    float part = 0.f, vf[kPerLane];
+  float m = kNegBig, l = 0.f;  // running maximum (wave uniform) and this lane's share of the sum
+  for (int j0 = wave * 32; j0 < context_len; j0 += kPaGenericWaves * 32) {
+    const int j = j0 + tok;
+    const bool live = j < context_len;
+    const int jc = live ? j : context_len - 1;  // dead lanes read a valid token and are masked
+    const int blk = jc / block_size;
+    const int64_t page = min(max(table[blk], 0), num_blocks - 1);
+    // offset of (token, kv head g, d-chunk row 0, this lane's half)
+    const int64_t base = ((page * row_chunks + (int64_t)g * chunks) * block_size + (jc - blk * block_size)) * 16 + 8 * half;
+    const int64_t chunk_stride = (int64_t)block_size * 16;
+    f16x8 kv[CH];
 #pragma unroll
-    for (int i = 0; i < kPerLane; ++i) {
-      const bool live = lane + kWave * i < head_dim;
-      part += live ? qf[i] * (float)key_cache[base + elem_off[i]] : 0.f;
-      vf[i] = live ? (float)value_cache[base + elem_off[i]] : 0.f;
-    }
-    const float sc = wave_sum(part) * scale_log2;
-    const float m_new = fmaxf(m, sc);
+    for (int c = 0; c < CH; ++c)
+      if (c < chunks) kv[c] = ld128_stream(key_cache + base + c * chunk_stride);
+    float part = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+      if (c < chunks) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) part += (float)qv[c][e] * (float)kv[c][e];
+      }
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+      if (c < chunks) kv[c] = ld128_stream(value_cache + base + c * chunk_stride);
+    part += __shfl_xor(part, 1);
+    const float sc = live ? part * scale_log2 : -__builtin_inff();
+    float mx = sc;
+#pragma unroll
+    for (int d = 2; d < kWave; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+    const float m_new = fmaxf(m, mx);  // finite: token j0 of the block is live
     const float alpha = __builtin_amdgcn_exp2f(m - m_new);
-    const float p = __builtin_amdgcn_exp2f(sc - m_new);
+    const float p = live ? __builtin_amdgcn_exp2f(sc - m_new) : 0.f;
     m = m_new;
     l = l * alpha + p;
 #pragma unroll
-    for (int i = 0; i < kPerLane; ++i) acc[i] = acc[i] * alpha + p * vf[i];
-  }
-  __shared__ float sm_acc[4][kPaGenericMaxD];
-  __shared__ float sm_m[4], sm_l[4];
+    for (int c = 0; c < CH; ++c)
+      if (c < chunks) {
 #pragma unroll
-  for (int i = 0; i < kPerLane; ++i) sm_acc[wave][lane + kWave * i] = acc[i];
+        for (int e = 0; e < 8; ++e) {
+          // cache contents of dead tokens are arbitrary (possibly NaN): they must not reach the sum
+          const float v = live ? (float)kv[c][e] : 0.f;
+          acc[c][e] = acc[c][e] * alpha + p * v;
+        }
+      }
+  }
+  // add up the 32 tokens of the wave (lanes with the same half), then the four waves
+  __shared__ float sm_acc[kPaGenericWaves][kPaGenericMaxD];
+  __shared__ float sm_m[kPaGenericWaves], sm_l[kPaGenericWaves];
+#pragma unroll
+  for (int d = 2; d < kWave; d <<= 1) l += __shfl_xor(l, d);
+#pragma unroll
+  for (int c = 0; c < CH; ++c)
+    if (c < chunks) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float v = acc[c][e];
+#pragma unroll
+        for (int d = 2; d < kWave; d <<= 1) v += __shfl_xor(v, d);
+        if (tok == 0) sm_acc[wave][16 * c + 8 * half + e] = v;
+      }
+    }
   if (lane == 0) {
     sm_m[wave] = m;
     sm_l[wave] = l;
   }
   __syncthreads();
-  for (int d = threadIdx.x; d < head_dim; d += 4 * kWave) {
+  for (int d = threadIdx.x; d < head_dim; d += kPaGenericWaves * kWave) {
     const float mx = fmaxf(fmaxf(sm_m[0], sm_m[1]), fmaxf(sm_m[2], sm_m[3]));
     float lsum = 0.f, a = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < kPaGenericWaves; ++w) {
       const float wt = __builtin_amdgcn_exp2f(sm_m[w] - mx);
       lsum += sm_l[w] * wt;
       a += sm_acc[w][d] * wt;
@@ -861,11 +910,14 @@ static int pa_run(const void* q, const void* key_cache, const void* value_cache,
   f16* op = static_cast<f16*>(o);
   if (!pa_fast_shape(num_heads, num_kv_heads, head_dim, block_size)) {
     const float scale_log2 = kLog2e / __builtin_sqrtf((float)head_dim);
-    dim3 grid((unsigned)num_heads, (unsigned)bs);
-    pa_decode_generic<<<grid, 4 * kWave, 0, s>>>(qp, kc, vc, block_tables, context_lens, op,
-                                                 (int)num_heads, (int)num_kv_heads, (int)head_dim,
-                                                 (int)block_size, (int)max_blocks_per_seq,
-                                                 scale_log2, (int)num_blocks);
+    const int64_t total = bs * num_heads;
+    const int64_t grid = (total + kPaXcds - 1) / kPaXcds * kPaXcds;
+    if (grid > 0x7fffffff) return AOPS_ERR_INVALID_ARGUMENT;
+    auto kernel = head_dim <= 64 ? pa_decode_generic<4> : head_dim <= 128 ? pa_decode_generic<8> : pa_decode_generic<16>;
+    kernel<<<(unsigned)grid, kPaGenericWaves * kWave, 0, s>>>(qp, kc, vc, block_tables, context_lens, op, (int)bs,
+                                                             (int)num_heads, (int)num_kv_heads, (int)head_dim,
+                                                             (int)block_size, (int)max_blocks_per_seq, scale_log2,
+                                                             (int)num_blocks);
     return record_launch_status(hipGetLastError());
   }
   const size_t need = aops_paged_attention_workspace(bs, num_heads, num_kv_heads, head_dim,

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ascend910a_extras operator set on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|norm|cache|rope|mlp|moe|pa_more|dense|scaled,...] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|norm|cache|rope|mlp|moe|moe_gate_up|moe_down|pa_more|dense|scaled,...] [--no-cpu]
 
 A "step" is one paged_attention decode call over the batch of BASELINE.json configs[4]
 (64 sequences, 32 query / 8 kv heads, head_dim 128, contexts ~U[512, 4096], block 128): the
@@ -561,6 +561,24 @@ def bench_moe(L, ops, R, dev, cpu):
     return out
 
 
+def bench_moe_one(L, ops, R, dev, which):
+    """One GEMM of configs[3] by itself (for profiler runs that must tell the two apart): gate_up on x ~ N(0,1),
+    or down on activations of the magnitude the real chain produces."""
+    import torch
+
+    E, hidden, inter, tokens, topk = 128, 2048, 768, 4096, 8
+    torch.manual_seed(0)
+    rows = tokens * topk
+    gl = R.make_group_list(torch.randint(0, E, (rows,)), E)
+    K, N = (hidden, 2 * inter) if which == "gate_up" else (inter, hidden)
+    x = (torch.randn(rows, K) * (1.0 if which == "gate_up" else 0.3)).half()
+    w = torch.empty(E, N, K, dtype=torch.float16)
+    for e in range(E):
+        w[e] = (0.02 * torch.randn(N, K)).half()
+    e, _ = _gmm_entry(L, ops, R, dev, False, "grouped_matmul", f"4: MoE {which} (alone)", x, w, gl)
+    return e
+
+
 def bench_mlp(L, ops, R, dev, cpu):
     import torch
 
@@ -822,6 +840,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--ops", default="all", help="comma list of: pa,norm,cache,mlp,moe,rope,scaled or all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--skip-headline", action="store_true",
+                    help="profiler runs of single operators: do not run the paged-attention headline workload "
+                         "(the last line then carries the per-operator records only)")
     ap.add_argument("--calib", action="store_true",
                     help="also run a plain elementwise copy of 512 MiB (reads 512 MiB, writes 512 MiB): the known-size "
                          "kernel against which FETCH_SIZE / WRITE_SIZE counters of a profiler run are scaled")
@@ -867,6 +888,16 @@ def main():
             log(f"[bench] {tag} done in {time.perf_counter() - t0:.1f}s")
             torch.cuda.empty_cache()
 
+    if args.skip_headline:
+        for tag, fn in (("moe_gate_up", lambda: bench_moe_one(L, ops, R, dev, "gate_up")),
+                        ("moe_down", lambda: bench_moe_one(L, ops, R, dev, "down")),
+                        ("dense", lambda: bench_dense(L, R, dev)),
+                        ("pa_more", lambda: bench_pa_more(L, R, dev, cpu))):
+            if tag in want:
+                run(tag, fn)
+        print(json.dumps({"per_op": per_op}), flush=True)
+        return
+
     # ------------------------------------------------------------------ primary: paged attention
     t0 = time.perf_counter()
     wl = PagedAttentionWorkload(R, dev)
@@ -892,6 +923,10 @@ def main():
     run("rope", lambda: bench_rope(L, ops, R, dev, cpu, 64, "5: rope", floor=True))
     run("mlp", lambda: bench_mlp(L, ops, R, dev, cpu))
     run("moe", lambda: bench_moe(L, ops, R, dev, cpu))
+    if "moe_gate_up" in want:
+        run("moe_gate_up", lambda: bench_moe_one(L, ops, R, dev, "gate_up"))
+    if "moe_down" in want:
+        run("moe_down", lambda: bench_moe_one(L, ops, R, dev, "down"))
     run("pa_more", lambda: bench_pa_more(L, R, dev, cpu))
     run("dense", lambda: bench_dense(L, R, dev))
     run("scaled", lambda: [
