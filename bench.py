@@ -816,20 +816,22 @@ def kernel_source_digest():
     return h.hexdigest()[:16]
 
 
+PER_KERNEL_FIELDS = ["op", "config", "us", "frac_of_peak", "bound", "launch_floor_us", "cpu_ms"]
+_SHORT = {"grouped_matmul": "gmm", "grouped_matmul_swiglu": "gmm+swiglu", "grouped_matmul_swiglu_gather": "gmm+swiglu+gather",
+          "paged_attention": "pa", "reshape_and_cache": "cache", "add_rms_norm": "norm"}
+
+
 def compact(e):
-    """One per_kernel record of the headline: operator, config, time, fraction of the bounding peak, CPU ms."""
+    """One per_kernel row of the headline, in the order of PER_KERNEL_FIELDS (a list keeps the line short)."""
     if "error" in e:
-        return {"op": e.get("op_group"), "error": e["error"][:80]}
+        return [e.get("op_group"), "error: " + e["error"][:60]]
     frac = e.get("mfma_frac") if e.get("bound") == "mfma" else e.get("hbm_frac")
-    c = {"op": e["op"], "config": e["config"].split(":")[0][:24], "us": round(e["gpu_us"], 1), "bound": e.get("bound"),
-         "frac": frac}
-    if "TFLOPs" in e and e.get("bound") == "mfma":
-        c["TFLOPs"] = e["TFLOPs"]
-    if "launch_floor_us" in e:
-        c["floor_us"] = e["launch_floor_us"]
-    if "cpu_ms" in e:
-        c["cpu_ms"] = round(e["cpu_ms"], 1)
-    return c
+    cfg = e["config"]
+    for cut in (" (", ": add", ": resh", ": rope", ": MLP"):
+        cfg = cfg.split(cut)[0]
+    cpu = e.get("cpu_ms")
+    return [_SHORT.get(e["op"], e["op"]), cfg[:34], round(e["gpu_us"], 1), None if frac is None else round(frac, 3),
+            e.get("bound"), e.get("launch_floor_us"), None if cpu is None else round(cpu, 1)]
 
 
 # --------------------------------------------------------------------------------------- main
@@ -973,9 +975,14 @@ def main():
     # the full per-operator records on their own line, BEFORE the headline (which must be the last line)
     print(json.dumps({"per_op": per_op}), flush=True)
 
-    wanted = ("1:", "2:", "3: MLP swiglu", "5: rope", "4: MoE gate_up", "4: MoE down", "4: MoE gate_up + down",
-              "4: MoE gate_up + activation, fused", "5 at batch 8", "5 at batch 1", "5 skewed: 64", "dense 8192")
-    per_kernel = [compact(e) for e in per_op if "error" in e or any(e.get("config", "").startswith(w) for w in wanted)]
+    wanted = ("1:", "2:", "3: MLP swiglu", "5: rope", "4: MoE gate_up", "4: MoE down", "5 at batch 8", "5 at batch 1",
+              "5 skewed: 64", "dense 8192")
+    unwanted = ("4: MoE gate_up + down", "4: MoE gate_up + activation + row gather")
+    per_kernel = [compact(e) for e in per_op
+                  if "error" in e or (any(e.get("config", "").startswith(w) for w in wanted)
+                                      and not any(e.get("config", "").startswith(u) for u in unwanted))]
+    if traffic_note and traffic is None:
+        log(f"[bench] roofline.traffic: {traffic_note}")
     gmm_sum = next((e for e in per_op if e.get("config", "").startswith("4: MoE gate_up + down")), None)
     gmm_cpu = [e.get("cpu_ms") for e in per_op if e.get("config") in ("4: MoE gate_up", "4: MoE down")]
 
@@ -996,7 +1003,6 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "BASELINE configs[4]: paged-attention decode, B=64, 32q/8kv heads, D=128, block 128, ctx~U[512,4096]",
-            "value_is": "paged-attention algorithmic bytes / wall step through the Python API",
             "sum_context_tokens": sum_ctx,
             "algorithmic_bytes_per_step": alg_bytes,
         },
@@ -1007,14 +1013,14 @@ def main():
             "unit": "GB/s",
             "frac": round(gbps_kernel / HBM_PEAK_GBPS, 4),
             "traffic": traffic,
-            "traffic_note": traffic_note,
             "kernel": "pa_decode_partial<128,4,true>",
             "us_per_call": pa["gpu_us"],
             "gmm": None if not gmm_sum else {
-                "config": "BASELINE configs[3] gate_up + down", "bound": "mfma", "TFLOPs": gmm_sum["TFLOPs"],
-                "peak": MFMA_F16_PEAK_TFLOPS, "frac": gmm_sum["mfma_frac"], "us": gmm_sum["gpu_us"],
+                "config": "configs[3] gate_up+down", "bound": "mfma", "TFLOPs": gmm_sum["TFLOPs"],
+                "peak": MFMA_F16_PEAK_TFLOPS, "frac": gmm_sum["mfma_frac"], "us": round(gmm_sum["gpu_us"], 1),
                 "cpu_ms": None if not all(gmm_cpu) or len(gmm_cpu) != 2 else round(sum(gmm_cpu), 1),
             },
+            "per_kernel_fields": PER_KERNEL_FIELDS,
             "per_kernel": per_kernel,
         },
         "cpu_baseline": None if not cpu else {
@@ -1022,7 +1028,7 @@ def main():
             "unit": "GB/s",
             "cores": cores,
             "kind": "port",
-            "sample": "the full configs[4] batch (64 sequences); torch fp32 oracle",
+            "sample": "full configs[4] batch; torch fp32 oracle",
             "runs": f"1 warm-up + median of {CPU_RUNS}",
             "ms": pa["cpu_ms"],
         },
