@@ -122,14 +122,15 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   const f16* b_base;
   const int lane_row = wave * 8 + ((lane >> 3) ^ (wave & 1));
   const int lane_c = (lane & 7) ^ (lane_row & 7);
-  const uint32_t off0 = (uint32_t)lane_row * (uint32_t)k + lane_c * 8;
-  const uint32_t copy_stride = 8u * kWaves * (uint32_t)k;
+  // per-lane offsets of the copies, in bytes (320 rows of at most 2^22 elements: below 2^32)
+  const uint32_t off0 = ((uint32_t)lane_row * (uint32_t)k + lane_c * 8) * 2u;
+  const uint32_t copy_stride = 8u * kWaves * (uint32_t)k * 2u;
   uint32_t a_last, b_last;  // offset of this lane's chunk in the last valid row
   uint32_t a_src[GATHER ? kACopies : 1];  // GATHER: offset of this lane's chunk per copy
   // SWIGLU: copy i of the weights fills row blocks 2i (gate rows 32i..32i+31 of the item) and
   // 2i+1 (the up rows d further down): per-lane offset + 32 rows per copy; b_last then holds the
   // number of valid 32-column blocks of the item instead of an offset.
-  const uint32_t off0_glu = ((uint32_t)(lane_row & 31) + (lane_row >= 32 ? (uint32_t)n_out : 0u)) * (uint32_t)k + lane_c * 8;
+  const uint32_t off0_glu = (((uint32_t)(lane_row & 31) + (lane_row >= 32 ? (uint32_t)n_out : 0u)) * (uint32_t)k + lane_c * 8) * 2u;
   auto set_sources = [&](const GmmWork& it) {
     const int lane_s = lane_id_fresh();
     const int lane_row = wave * 8 + ((lane_s >> 3) ^ (wave & 1));
@@ -144,18 +145,18 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
         const int r = min(8 * kWaves * i + lane_row, x_left - 1);
         uint32_t src = (uint32_t)row_idx[it.row_begin + r] / (uint32_t)idx_div;
         src = src < x_rows ? src : x_rows - 1;  // an index outside x reads its last row instead of faulting
-        a_src[i] = src * (uint32_t)k + lane_c * 8;
+        a_src[i] = src * (uint32_t)k + lane_c * 8;  // in elements: up to 2^32 of them
       }
     } else {
       a_base = x + (int64_t)it.row_begin * k;
     }
-    a_last = (uint32_t)(x_left - 1) * (uint32_t)k + lane_c * 8;
-    b_last = SWIGLU ? (uint32_t)(n_left / 32) : (uint32_t)(n_left - 1) * (uint32_t)k + lane_c * 8;
+    a_last = ((uint32_t)(x_left - 1) * (uint32_t)k + lane_c * 8) * 2u;
+    b_last = SWIGLU ? (uint32_t)(n_left / 32) : ((uint32_t)(n_left - 1) * (uint32_t)k + lane_c * 8) * 2u;
   };
   auto b_offset = [&](int i) -> uint32_t {
     if constexpr (SWIGLU) {
       const uint32_t blk = (uint32_t)i < b_last ? (uint32_t)i : 0u;  // blocks past n: repeat block 0
-      return off0_glu + blk * 32u * (uint32_t)k;
+      return off0_glu + blk * 64u * (uint32_t)k;
     } else {
       return min(off0 + i * copy_stride, b_last);
     }
@@ -164,20 +165,29 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     const int ko = kt * kBK;
     f16* da = sa + stage * BM * kBK + wave * 512;
     f16* db = sb + stage * BN * kBK + wave * 512;
-    // the empty asm makes the 64-bit source address of a copy be formed right before the copy
-    // instead of being kept in a register pair per copy across the k loop
 #pragma unroll
     for (int i = 0; i < kACopies; ++i) {
-      uint32_t o = GATHER ? a_src[i] : min(off0 + i * copy_stride, a_last);
-      asm volatile("" : "+v"(o));
-      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(a_base + ko + o),
-                                       AOPS_LDS_PTR(da + i * kWaves * 512), 16, 0, 0);
+      if constexpr (GATHER) {  // offsets of up to 2^32 elements: 64-bit address arithmetic
+        // (the empty asm makes the 64-bit source address be formed right before the copy instead of being
+        // kept in a register pair per copy across the k loop)
+        uint32_t o = a_src[i];
+        asm volatile("" : "+v"(o));
+        __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(a_base + ko + o),
+                                         AOPS_LDS_PTR(da + i * kWaves * 512), 16, 0, 0);
+      } else {
+        // uniform base + 32-bit byte offset per lane: the copy takes them as they are (scalar base,
+        // vector offset), no vector instructions spent on a 64-bit address
+        const uint32_t o = min(off0 + i * copy_stride, a_last);
+        const char* ab = reinterpret_cast<const char*>(a_base + ko);
+        __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(ab + (uint64_t)o),
+                                         AOPS_LDS_PTR(da + i * kWaves * 512), 16, 0, 0);
+      }
     }
 #pragma unroll
     for (int i = 0; i < kBCopies; ++i) {
-      uint32_t o = b_offset(i);
-      asm volatile("" : "+v"(o));
-      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(b_base + ko + o),
+      const uint32_t o = b_offset(i);
+      const char* bb = reinterpret_cast<const char*>(b_base + ko);
+      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(bb + (uint64_t)o),
                                        AOPS_LDS_PTR(db + i * kWaves * 512), 16, 0, 0);
     }
   };
@@ -185,9 +195,16 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   const int fm = lane & 31;
   const int fq = lane >> 5;
   // Fragment addresses: lds_off(fm, 2*st + fq) == lds_off(fm, fq) ^ (st << 4) (the k step only
-  // flips two chunk bits), so one per-lane offset per operand serves every k step.
-  const int fa_off0 = lds_off(fm, fq) + wm * 32 * kBK;
-  const int fb_off0 = lds_off(fm, fq) + wn * 32 * NB * kBK;
+  // flips two chunk bits), so one LDS byte address per operand and stage serves every k step: the
+  // step's XOR is one vector instruction, row block and column block are immediate offsets of the
+  // reads.  (Both regions start on 128-byte boundaries, so the XOR of bits 5-6 stays inside a row.)
+  typedef const __attribute__((address_space(3))) f16x8* LdsFrag;
+  const uint32_t lds_sa = (uint32_t)(uintptr_t)AOPS_LDS_PTR(sa);
+  const uint32_t lds_sb = (uint32_t)(uintptr_t)AOPS_LDS_PTR(sb);
+  const uint32_t fa_byte0 = lds_sa + (uint32_t)(lds_off(fm, fq) + wm * 32 * kBK) * 2u;
+  const uint32_t fb_byte0 = lds_sb + (uint32_t)(lds_off(fm, fq) + wn * 32 * NB * kBK) * 2u;
+  const uint32_t fa_byte[2] = {fa_byte0, fa_byte0 + BM * kBK * 2u};
+  const uint32_t fb_byte[2] = {fb_byte0, fb_byte0 + BN * kBK * 2u};
 
   f32x16 acc[MB][NB];
   GmmWork nxt;
@@ -195,28 +212,30 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   auto k_loop = [&](auto live_c) {
     constexpr int LIVE = decltype(live_c)::value;
     f16x8 fa[2][LIVE > 0 ? LIVE : 1], fb[2][NB];
-    auto load_frags = [&](int buf, int st, int stage) {
-      // the empty asm keeps the compiler from hoisting one address register per (stage, step)
-      // out of the k loop, which would push the accumulators into scratch
-      int fo_a = fa_off0, fo_b = fb_off0;
-      asm volatile("" : "+v"(fo_a), "+v"(fo_b));
-      const f16* ca = sa + stage * BM * kBK + (fo_a ^ (st << 4));
-      const f16* cb = sb + stage * BN * kBK + (fo_b ^ (st << 4));
+    auto load_frags = [&](int buf, auto st_c, auto stage_c) {
+      constexpr int ST = decltype(st_c)::value;
+      constexpr int STAGE = decltype(stage_c)::value;
+      // The XOR is a volatile asm: written as an expression it would be hoisted out of the k loop, one
+      // address register per (operand, stage, step), and push the accumulators into scratch.
+      uint32_t pa = fa_byte[STAGE], pb = fb_byte[STAGE];
+      if constexpr (ST > 0) {
+        asm volatile("v_xor_b32 %0, %1, %2" : "=v"(pa) : "n"(ST << 5), "v"(fa_byte[STAGE]));
+        asm volatile("v_xor_b32 %0, %1, %2" : "=v"(pb) : "n"(ST << 5), "v"(fb_byte[STAGE]));
+      }
 #pragma unroll
-      for (int j = 0; j < NB; ++j)
-        fb[buf][j] = *reinterpret_cast<const f16x8*>(&cb[j * 32 * kBK]);
+      for (int j = 0; j < NB; ++j) fb[buf][j] = *reinterpret_cast<LdsFrag>(pb + j * 32 * kBK * 2);
 #pragma unroll
-      for (int i = 0; i < LIVE; ++i)
-        fa[buf][i] = *reinterpret_cast<const f16x8*>(&ca[i * 64 * kBK]);
+      for (int i = 0; i < LIVE; ++i) fa[buf][i] = *reinterpret_cast<LdsFrag>(pa + i * 64 * kBK * 2);
     };
     auto step = [&](int kcopy, auto stage_c, auto st_c) {
       constexpr int STAGE = decltype(stage_c)::value;
       constexpr int ST = decltype(st_c)::value;
-      if (ST + 1 < kSteps) {
-        load_frags((ST + 1) & 1, ST + 1, STAGE);
+      if constexpr (ST + 1 < kSteps) {
+        load_frags((ST + 1) & 1, std::integral_constant<int, ST + 1>{}, stage_c);
       } else {
-        load_frags(0, 0, STAGE ^ 1);  // first fragments of the next tile
-        copy_tile(kcopy, STAGE);      // this stage is free: everyone is past the barrier
+        // first fragments of the next tile
+        load_frags(0, std::integral_constant<int, 0>{}, std::integral_constant<int, STAGE ^ 1>{});
+        copy_tile(kcopy, STAGE);  // this stage is free: everyone is past the barrier
       }
 #pragma unroll
       for (int i = 0; i < LIVE; ++i)
@@ -242,7 +261,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     };
     using I0 = std::integral_constant<int, 0>;
     using I1 = std::integral_constant<int, 1>;
-    load_frags(0, 0, 0);
+    load_frags(0, I0{}, I0{});
     for (int kt = 0; kt < ktiles; kt += 2) {
       int c0 = kt + 2, c1 = kt + 3;
       if (kt + 2 >= ktiles) {  // the last two tiles fetch the head of the next item
