@@ -55,10 +55,23 @@ extern "C" int aops_swiglu_f16(const void* x, void* y, int64_t num_tokens, int64
   const int64_t vec_per_row = d / 8;
   const int64_t total = num_tokens * vec_per_row;
   if (total >= ((int64_t)1 << 32) - 4096) return AOPS_ERR_INVALID_ARGUMENT;
-  constexpr int kUnroll = 2;
-  const unsigned grid = (unsigned)((total + 256 * kUnroll - 1) / (256 * kUnroll));
-  swiglu_kernel<kUnroll><<<grid, 256, 0, static_cast<hipStream_t>(stream)>>>(
-      static_cast<const f16*>(x), static_cast<f16*>(y), (uint32_t)total, (uint32_t)vec_per_row,
-      d);
+  // Vectors per thread: two (measured best on large inputs; four is 5-8 % slower), or one when that
+  // leaves the fullest CU less to do.  Small inputs are resident all at once, workgroups dealt round robin,
+  // so the time is that of the fullest CU: 896 workgroups of two vectors per thread give 256 CUs three or
+  // four each (12 % above the mean), 1792 of one vector give every CU seven ([256, 28672]: 6.1 -> 5.2 us).
+  const int64_t cus = device_cu_count();
+  auto fullest = [&](int u) {  // vectors per thread slot of the CU with the most workgroups
+    const int64_t wgs = (total + 256 * u - 1) / (256 * u);
+    return (wgs + cus - 1) / cus * u;
+  };
+  const int unroll = fullest(1) < fullest(2) ? 1 : 2;
+  const unsigned grid = (unsigned)((total + 256 * unroll - 1) / (256 * unroll));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const f16* xp = static_cast<const f16*>(x);
+  f16* yp = static_cast<f16*>(y);
+  if (unroll == 2)
+    swiglu_kernel<2><<<grid, 256, 0, s>>>(xp, yp, (uint32_t)total, (uint32_t)vec_per_row, d);
+  else
+    swiglu_kernel<1><<<grid, 256, 0, s>>>(xp, yp, (uint32_t)total, (uint32_t)vec_per_row, d);
   return record_launch_status(hipGetLastError());
 }
