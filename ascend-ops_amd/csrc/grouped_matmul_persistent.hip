@@ -327,7 +327,8 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
       constexpr int kRowsPerUnit = kEpiScratchHalfs / kSegHalfs;  // 8 rows of 128 bytes, or 16 of 64
       constexpr int kSlots = kSegHalfs / 8;                  // 16-byte slots per row segment
       constexpr int kUnits = 32 / kRowsPerUnit;
-      static_assert(kSegHalfs == 64 || kSegHalfs == 32, "row segment of 128 or 64 bytes");
+      static_assert(kSegHalfs == 128 || kSegHalfs == 64 || kSegHalfs == 32, "row segment of 256, 128 or 64 bytes");
+      static_assert(kRowsPerUnit <= 32 && 32 % kRowsPerUnit == 0 && kRowsPerUnit * kSlots == kWave, "one 16-byte slot per lane");
       const int col_w = SWIGLU ? cur.n_tile * BNO + wn * 32 : cur.n_tile * BN + wn * 32 * NB;
       // the lane-derived offsets are the same for every item; taken from a fresh lane id they are not
       // hoisted out of the item loop (and spilled)
@@ -339,7 +340,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
       const int r_r = lane_e / kSlots;                        // the row this lane reads back and stores
       const int q_r = lane_e % kSlots;                        // ... and its 16-byte slot
       // slot swizzle of row r: rows whose segments start in the same bank get different slot orders
-      auto swz = [](int r) { return kSlots == 8 ? (r & 7) : ((r ^ (r >> 2)) & 3); };
+      auto swz = [](int r) { return kSlots == 16 ? (r & 3) : kSlots == 8 ? (r & 7) : ((r ^ (r >> 2)) & 3); };
       const f16* rd = scr + r_r * kSegHalfs + ((q_r ^ swz(r_r)) * 8);
 #pragma unroll
       for (int i = 0; i < MB; ++i) {
