@@ -6,11 +6,13 @@ namespace aops {
 
 // Persistent form of grouped_matmul_dma_kernel: one workgroup per CU walks through its share of
 // the work items (XCD x owns a contiguous range of items, its workgroups take them round robin),
-// and the operand pipeline never drains between items: the last two k tiles of an item issue the
-// copies of the first two tiles of the next item, and the finished accumulators leave straight
-// from registers (lane pairs exchange halves with v_permlane32_swap so that every lane stores 16
-// contiguous bytes) while those copies are in flight, with no LDS use and no workgroup barrier.
-// group_list is scanned once per workgroup; every wave keeps its copy of the scan in LDS.
+// and the operand pipeline never drains between items: the last tiles of an item issue the copies
+// of the first tiles of the next item (its weights two tiles ahead, its activation rows one), and
+// the finished accumulators leave through a small LDS scratch of the wave's own while those copies
+// are in flight, with no workgroup barrier.  The two operands have separate two-stage rings: the
+// weight stage of a tile is free as soon as every wave holds its fragments in registers (barrier B
+// of the k loop), the activation stage when the tile's last fragment has been read (barrier A).
+// group_list is scanned once per workgroup; the scan is kept in LDS.
 // Requires k % 128 == 0 and k >= 256 (an even number of k tiles keeps the stage parity fixed).
 //
 // SWIGLU = true fuses the activation of a gate_up projection into the epilogue: with d = n/2 the
@@ -34,6 +36,27 @@ __device__ __forceinline__ int lane_id_fresh() {
   asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
   return l;
 }
+
+// Operand copy HBM/L2 -> LDS, 16 bytes per lane: lane l's bytes land at LDS byte address lds_addr + 16*l.
+// Written as inline asm rather than through the compiler's builtin: the compiler's wait-count pass treats
+// the builtin as an access to both memory and LDS and, while one is outstanding, turns every wait for an
+// LDS read into a wait for all of them - and this kernel always has copies outstanding.  The kernel waits
+// for its copies itself (counted s_waitcnt vmcnt before the barriers); the asm is invisible to that pass,
+// which errs on the safe side for the loads and stores it does see (invisible operations only make a
+// counted wait stricter, never looser, since vector memory operations complete in order).
+// M0 carries the LDS address of a copy; the compiler reserves that register and warns when it appears in a
+// clobber list, but nothing else in this kernel uses it.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void dma16(const void* base, uint32_t lane_offset, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :: "s"(lds_addr), "v"(lane_offset), "s"(base) : "m0", "memory");
+}
+__device__ __forceinline__ void dma16(const void* lane_address, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :: "s"(lds_addr), "v"(lane_address) : "m0", "memory");
+}
+#pragma clang diagnostic pop
 
 constexpr int kPlanInts = 2 + kBndCache + 1;  // per-lane record of the group_list scan kept in LDS
 constexpr int kEpiScratchHalfs = 512;         // 1 KiB of LDS per wave for the epilogue's row transposition
@@ -131,12 +154,18 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   // 2i+1 (the up rows d further down): per-lane offset + 32 rows per copy; b_last then holds the
   // number of valid 32-column blocks of the item instead of an offset.
   const uint32_t off0_glu = (((uint32_t)(lane_row & 31) + (lane_row >= 32 ? (uint32_t)n_out : 0u)) * (uint32_t)k + lane_c * 8) * 2u;
-  auto set_sources = [&](const GmmWork& it) {
+  auto set_w_sources = [&](const GmmWork& it) {
     const int lane_s = lane_id_fresh();
     const int lane_row = wave * 8 + ((lane_s >> 3) ^ (wave & 1));
     const int lane_c = (lane_s & 7) ^ (lane_row & 7);
     b_base = w + ((int64_t)it.expert * n + (int64_t)it.n_tile * BNO) * k;
     const int n_left = min(n_out - it.n_tile * BNO, BNO);
+    b_last = SWIGLU ? (uint32_t)(n_left / 32) : ((uint32_t)(n_left - 1) * (uint32_t)k + lane_c * 8) * 2u;
+  };
+  auto set_x_sources = [&](const GmmWork& it) {
+    const int lane_s = lane_id_fresh();
+    const int lane_row = wave * 8 + ((lane_s >> 3) ^ (wave & 1));
+    const int lane_c = (lane_s & 7) ^ (lane_row & 7);
     const int x_left = min(it.row_end - it.row_begin, BM);  // rows of the group in this tile
     if constexpr (GATHER) {
       a_base = x;
@@ -151,7 +180,6 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
       a_base = x + (int64_t)it.row_begin * k;
     }
     a_last = ((uint32_t)(x_left - 1) * (uint32_t)k + lane_c * 8) * 2u;
-    b_last = SWIGLU ? (uint32_t)(n_left / 32) : ((uint32_t)(n_left - 1) * (uint32_t)k + lane_c * 8) * 2u;
   };
   auto b_offset = [&](int i) -> uint32_t {
     if constexpr (SWIGLU) {
@@ -161,35 +189,27 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
       return min(off0 + i * copy_stride, b_last);
     }
   };
-  auto copy_tile = [&](int kt, int stage) {
+  const uint32_t lds_sa = (uint32_t)(uintptr_t)AOPS_LDS_PTR(sa);  // LDS byte addresses of the stages
+  const uint32_t lds_sb = (uint32_t)(uintptr_t)AOPS_LDS_PTR(sb);
+  auto copy_x = [&](int kt, int stage) {
     const int ko = kt * kBK;
-    f16* da = sa + stage * BM * kBK + wave * 512;
-    f16* db = sb + stage * BN * kBK + wave * 512;
+    const uint32_t da = lds_sa + (uint32_t)(stage * BM * kBK + wave * 512) * 2u;
 #pragma unroll
     for (int i = 0; i < kACopies; ++i) {
-      if constexpr (GATHER) {  // offsets of up to 2^32 elements: 64-bit address arithmetic
-        // (the empty asm makes the 64-bit source address be formed right before the copy instead of being
-        // kept in a register pair per copy across the k loop)
-        uint32_t o = a_src[i];
-        asm volatile("" : "+v"(o));
-        __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(a_base + ko + o),
-                                         AOPS_LDS_PTR(da + i * kWaves * 512), 16, 0, 0);
+      if constexpr (GATHER) {  // offsets of up to 2^32 elements: 64-bit address per lane
+        dma16(a_base + ko + a_src[i], da + i * kWaves * 1024);
       } else {
         // uniform base + 32-bit byte offset per lane: the copy takes them as they are (scalar base,
         // vector offset), no vector instructions spent on a 64-bit address
-        const uint32_t o = min(off0 + i * copy_stride, a_last);
-        const char* ab = reinterpret_cast<const char*>(a_base + ko);
-        __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(ab + (uint64_t)o),
-                                         AOPS_LDS_PTR(da + i * kWaves * 512), 16, 0, 0);
+        dma16(a_base + ko, min(off0 + i * copy_stride, a_last), da + i * kWaves * 1024);
       }
     }
+  };
+  auto copy_w = [&](int kt, int stage) {
+    const int ko = kt * kBK;
+    const uint32_t db = lds_sb + (uint32_t)(stage * BN * kBK + wave * 512) * 2u;
 #pragma unroll
-    for (int i = 0; i < kBCopies; ++i) {
-      const uint32_t o = b_offset(i);
-      const char* bb = reinterpret_cast<const char*>(b_base + ko);
-      __builtin_amdgcn_global_load_lds(AOPS_GLOBAL_PTR(bb + (uint64_t)o),
-                                       AOPS_LDS_PTR(db + i * kWaves * 512), 16, 0, 0);
-    }
+    for (int i = 0; i < kBCopies; ++i) dma16(b_base + ko, b_offset(i), db + i * kWaves * 1024);
   };
 
   const int fm = lane & 31;
@@ -199,8 +219,6 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   // step's XOR is one vector instruction, row block and column block are immediate offsets of the
   // reads.  (Both regions start on 128-byte boundaries, so the XOR of bits 5-6 stays inside a row.)
   typedef const __attribute__((address_space(3))) f16x8* LdsFrag;
-  const uint32_t lds_sa = (uint32_t)(uintptr_t)AOPS_LDS_PTR(sa);
-  const uint32_t lds_sb = (uint32_t)(uintptr_t)AOPS_LDS_PTR(sb);
   const uint32_t fa_byte0 = lds_sa + (uint32_t)(lds_off(fm, fq) + wm * 32 * kBK) * 2u;
   const uint32_t fb_byte0 = lds_sb + (uint32_t)(lds_off(fm, fq) + wn * 32 * NB * kBK) * 2u;
   const uint32_t fa_byte[2] = {fa_byte0, fa_byte0 + BM * kBK * 2u};
@@ -209,80 +227,135 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   f32x16 acc[MB][NB];
   GmmWork nxt;
 
+  // The k loop.  Per k tile t (stage t & 1) a wave reads its weight fragments of all four k steps into
+  // registers at once and its activation fragments one at a time, row block by row block:
+  //
+  //   barrier A(t): tile t has landed, nobody reads the activation stage of tile t-1 any more
+  //     -> activation copies of tile t+1, fragment reads of tile t between the last eight MFMAs of tile t-1
+  //   barrier B(t): everybody holds the weight fragments of tile t in registers
+  //     -> weight copies of tile t+2 into the weight stage of tile t
+  //   MFMAs of tile t ...
+  //
+  // The weights are read once, so each of their requests goes to memory and is slow; the activation
+  // rows mostly hit in L2.  Freeing the weight stage at the start of the tile gives the slow requests
+  // almost two tile periods to arrive, and barrier A(t+1) waits only for copies that were issued a full
+  // period before: the L1's queue of pending requests (what bounds this kernel) still holds the weight
+  // requests of tile t+2 when the next burst arrives, instead of draining to empty at every barrier.
   auto k_loop = [&](auto live_c) {
     constexpr int LIVE = decltype(live_c)::value;
-    f16x8 fa[2][LIVE > 0 ? LIVE : 1], fb[2][NB];
-    auto load_frags = [&](int buf, auto st_c, auto stage_c) {
+    constexpr int NF = kSteps * LIVE;  // activation fragments (pairs of MFMAs) of a k tile
+    constexpr int kFa = 4;             // activation fragments in flight
+    f16x8 fa[LIVE > 0 ? kFa : 1], fb[kSteps][NB];
+    // The XORs are volatile asm: written as expressions they would be hoisted out of the k loop, one
+    // address register per (operand, stage, step), and push the accumulators into scratch.
+    auto read_fb = [&](auto st_c, auto stage_c) {
       constexpr int ST = decltype(st_c)::value;
       constexpr int STAGE = decltype(stage_c)::value;
-      // The XOR is a volatile asm: written as an expression it would be hoisted out of the k loop, one
-      // address register per (operand, stage, step), and push the accumulators into scratch.
-      uint32_t pa = fa_byte[STAGE], pb = fb_byte[STAGE];
-      if constexpr (ST > 0) {
-        asm volatile("v_xor_b32 %0, %1, %2" : "=v"(pa) : "n"(ST << 5), "v"(fa_byte[STAGE]));
-        asm volatile("v_xor_b32 %0, %1, %2" : "=v"(pb) : "n"(ST << 5), "v"(fb_byte[STAGE]));
-      }
+      uint32_t pb = fb_byte[STAGE];
+      if constexpr (ST > 0) asm volatile("v_xor_b32 %0, %1, %2" : "=v"(pb) : "n"(ST << 5), "v"(fb_byte[STAGE]));
 #pragma unroll
-      for (int j = 0; j < NB; ++j) fb[buf][j] = *reinterpret_cast<LdsFrag>(pb + j * 32 * kBK * 2);
-#pragma unroll
-      for (int i = 0; i < LIVE; ++i) fa[buf][i] = *reinterpret_cast<LdsFrag>(pa + i * 64 * kBK * 2);
+      for (int j = 0; j < NB; ++j) fb[ST][j] = *reinterpret_cast<LdsFrag>(pb + j * 32 * kBK * 2);
     };
-    auto step = [&](int kcopy, auto stage_c, auto st_c) {
+    auto read_fa = [&](auto n_c, auto stage_c) {  // fragment n = (row block n / kSteps, k step n % kSteps)
+      constexpr int N = decltype(n_c)::value;
       constexpr int STAGE = decltype(stage_c)::value;
-      constexpr int ST = decltype(st_c)::value;
-      if constexpr (ST + 1 < kSteps) {
-        load_frags((ST + 1) & 1, std::integral_constant<int, ST + 1>{}, stage_c);
-      } else {
-        // first fragments of the next tile
-        load_frags(0, std::integral_constant<int, 0>{}, std::integral_constant<int, STAGE ^ 1>{});
-        copy_tile(kcopy, STAGE);  // this stage is free: everyone is past the barrier
+      if constexpr (N >= 0 && N < NF) {
+        constexpr int ST = N % kSteps;
+        uint32_t pa = fa_byte[STAGE];
+        if constexpr (ST > 0) asm volatile("v_xor_b32 %0, %1, %2" : "=v"(pa) : "n"(ST << 5), "v"(fa_byte[STAGE]));
+        fa[N % kFa] = *reinterpret_cast<LdsFrag>(pa + (N / kSteps) * 64 * kBK * 2);
       }
-#pragma unroll
-      for (int i = 0; i < LIVE; ++i)
+    };
+    auto mma = [&](auto n_c) {
+      constexpr int N = decltype(n_c)::value;
+      if constexpr (N >= 0 && N < NF) {
 #pragma unroll
         for (int j = 0; j < NB; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ST & 1][j], fa[ST & 1][i],
-                                                             acc[i][j], 0, 0, 0);
-      MfmaInterleave<0, LIVE * NB, LIVE + NB, 0,
-                     (ST + 1 < kSteps) ? 0 : kACopies + kBCopies>::run();
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    auto iteration = [&](int kcopy, auto stage_c) {
-      step(kcopy, stage_c, std::integral_constant<int, 0>{});
-      step(kcopy, stage_c, std::integral_constant<int, 1>{});
-      step(kcopy, stage_c, std::integral_constant<int, 2>{});
-      // own copies of the next tile and all own fragment reads of this tile are complete ...
-      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
-      asm volatile("" ::: "memory");
-      __builtin_amdgcn_s_barrier();  // ... and so are everybody else's
-      asm volatile("" ::: "memory");
-      __builtin_amdgcn_sched_barrier(0);
-      step(kcopy, stage_c, std::integral_constant<int, 3>{});
-    };
-    using I0 = std::integral_constant<int, 0>;
-    using I1 = std::integral_constant<int, 1>;
-    load_frags(0, I0{}, I0{});
-    for (int kt = 0; kt < ktiles; kt += 2) {
-      int c0 = kt + 2, c1 = kt + 3;
-      if (kt + 2 >= ktiles) {  // the last two tiles fetch the head of the next item
-        if (nxt.valid) {
-          set_sources(nxt);
-          c0 = 0;
-          c1 = 1;
-        } else {  // nothing follows: repeat the last tile (valid memory, never consumed)
-          c0 = c1 = ktiles - 1;
-        }
+          acc[N / kSteps][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[N % kSteps][j], fa[N % kFa],
+                                                                      acc[N / kSteps][j], 0, 0, 0);
       }
-      iteration(c0, I0{});
-      iteration(c1, I1{});
+    };
+    auto fence = [] {
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    // MFMA pairs N .. END-1 of the tile, each followed by the read of the fragment that takes its place
+    auto pairs = [&](auto self, auto n_c, auto end_c, auto stage_c) {
+      constexpr int N = decltype(n_c)::value;
+      if constexpr (N < decltype(end_c)::value) {
+        mma(n_c);
+        read_fa(std::integral_constant<int, N + kFa>{}, stage_c);
+        __builtin_amdgcn_sched_barrier(0);
+        self(self, std::integral_constant<int, N + 1>{}, end_c, stage_c);
+      }
+    };
+    // The last kTail pairs of a tile run at the start of the next one, between its first fragment reads,
+    // so that the matrix cores have work while those reads are on their way.
+    constexpr int kTail = kSteps;  // = kFa: the tail holds the whole fragment ring and every weight step
+    // barrier B comes after this many pairs of the tile: the burst of reads at its start has returned by
+    // then, so the wait in front of the barrier costs nothing
+    constexpr int kPairsBeforeB = NF - kTail < 6 ? NF - kTail : 6;
+    auto tile = [&](auto stage_c, int kx, int kw, bool tail, bool switch_x, bool switch_w) {
+      constexpr int STAGE = decltype(stage_c)::value;
+      if (switch_x) set_x_sources(nxt);
+      copy_x(kx, STAGE ^ 1);
+      if constexpr (LIVE > 0) {
+        auto start = [&](auto q_c) {  // tail pair q of the previous tile, then the reads that reuse its registers
+          constexpr int Q = decltype(q_c)::value;
+          if (tail) mma(std::integral_constant<int, NF - kTail + Q>{});
+          read_fa(q_c, stage_c);
+          __builtin_amdgcn_sched_barrier(0);  // the counted wait in front of barrier B relies on this order
+          read_fb(q_c, stage_c);
+          __builtin_amdgcn_sched_barrier(0);
+        };
+        start(std::integral_constant<int, 0>{});
+        start(std::integral_constant<int, 1>{});
+        start(std::integral_constant<int, 2>{});
+        start(std::integral_constant<int, 3>{});
+        pairs(pairs, std::integral_constant<int, 0>{}, std::integral_constant<int, kPairsBeforeB>{}, stage_c);
+      }
+      // all own weight fragments of this tile are in registers (LDS serves a wave's reads in order, and only
+      // the kPairsBeforeB refills of the activation ring were issued after the last of them) ...
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(0xc07f | ((LIVE > 0 ? kPairsBeforeB : 0) << 8));  // lgkmcnt only
+      fence();
+      __builtin_amdgcn_s_barrier();  // ... and so are everybody else's: barrier B
+      fence();
+      if (switch_w) set_w_sources(nxt);
+      copy_w(kw, STAGE);
+      if constexpr (LIVE > 0)
+        pairs(pairs, std::integral_constant<int, kPairsBeforeB>{}, std::integral_constant<int, NF - kTail>{}, stage_c);
+      // own copies of the next tile (all but the weight copies just issued) and all own fragment reads of
+      // this tile are complete ...
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kBCopies));
+      fence();
+      __builtin_amdgcn_s_barrier();  // ... and so are everybody else's: barrier A of the next tile
+      fence();
+    };
+    for (int kt = 0; kt < ktiles; kt += 2) {
+      const bool last = kt + 2 >= ktiles;  // the last two tiles fetch the head of the next item
+      const bool follow = last && nxt.valid;
+      // nothing follows: repeat the last tile (valid memory, never consumed)
+      tile(std::integral_constant<int, 0>{}, kt + 1, last ? (follow ? 0 : ktiles - 1) : kt + 2, kt > 0, false, follow);
+      tile(std::integral_constant<int, 1>{}, last ? (follow ? 0 : ktiles - 1) : kt + 2,
+           last ? (follow ? 1 : ktiles - 1) : kt + 3, true, follow, false);
+    }
+    if constexpr (LIVE > 0) {
+      mma(std::integral_constant<int, NF - 4>{});
+      mma(std::integral_constant<int, NF - 3>{});
+      mma(std::integral_constant<int, NF - 2>{});
+      mma(std::integral_constant<int, NF - 1>{});
     }
   };
 
-  set_sources(cur);
-  copy_tile(0, 0);
-  copy_tile(1, 1);
-  // tile 0 must be complete, tile 1 may still be on its way
-  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kACopies + kBCopies));
+  set_w_sources(cur);
+  set_x_sources(cur);
+  copy_w(0, 0);
+  copy_x(0, 0);
+  copy_w(1, 1);
+  // tile 0 must be complete, the weights of tile 1 may still be on their way
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kBCopies));
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
