@@ -728,25 +728,27 @@ static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t*
 }
 
 // Generic path for every other shape (head_dim a multiple of 16 up to 256, any block size, any
-// whole number of query heads per kv head): one workgroup of four waves per (sequence, query head).
-// A wave takes every fourth block of 32 tokens; lane (token = lane / 2, half = lane % 2) loads, d-chunk
+// whole number of query heads per kv head): one workgroup of eight waves per (sequence, query head).
+// A wave takes every eighth block of 32 tokens; lane (token = lane / 2, half = lane % 2) loads, d-chunk
 // row by d-chunk row, the 16 bytes that hold d = 16c + 8*half ..+7 of its token, so that a load
 // instruction of a wave covers 1 KiB of consecutive tokens of one d-chunk row (tokens of one page are
 // adjacent in the layout).  Scores are finished with one exchange between the two lanes of a token, the
 // block's softmax with wave reductions; every lane accumulates p * V for its own token and half, and the
-// 32 tokens are added up with lane exchanges once per wave at the end.  The four waves meet in LDS.
+// 32 tokens are added up with lane exchanges once per wave at the end.  The eight waves meet in LDS.
 // Workgroups are renumbered so that the query heads of one kv head, which read the same K and V, run on
 // one XCD side by side and share its L2.  CH = number of d-chunk rows the registers are sized for.
 constexpr int kPaGenericMaxD = 256;
-constexpr int kPaGenericWaves = 4;
+// eight waves where a wave's registers allow two waves per SIMD (head_dim <= 128), four otherwise
+constexpr int pa_generic_waves(int ch) { return ch <= 8 ? 8 : 4; }
 
 template <int CH>
-__global__ __launch_bounds__(kPaGenericWaves* kWave) void pa_decode_generic(
+__global__ __launch_bounds__(pa_generic_waves(CH) * kWave) void pa_decode_generic(
     const f16* __restrict__ q, const f16* __restrict__ key_cache,
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ context_lens, f16* __restrict__ out, int bs, int num_heads,
     int num_kv_heads, int head_dim, int block_size, int max_blocks_per_seq, float scale_log2,
     int num_blocks) {
+  constexpr int kPaGenericWaves = pa_generic_waves(CH);
   // XCD x takes the contiguous range [x * share, (x + 1) * share) of the (sequence, head) pairs
   const int total = bs * num_heads;
   const int share = (total + kPaXcds - 1) / kPaXcds;
@@ -774,29 +776,61 @@ __global__ __launch_bounds__(kPaGenericWaves* kWave) void pa_decode_generic(
     for (int e = 0; e < 8; ++e) acc[c][e] = 0.f;
   }
   float m = kNegBig, l = 0.f;  // running maximum (wave uniform) and this lane's share of the sum
-  for (int j0 = wave * 32; j0 < context_len; j0 += kPaGenericWaves * 32) {
+  const int64_t chunk_stride = (int64_t)block_size * 16;
+  // (token of this lane in the block that starts at j0) -> is it inside the context, and where its row starts:
+  // offset of (token, kv head g, d-chunk row 0, this lane's half).  Dead lanes read a valid token and are masked.
+  auto locate = [&](int j0, bool& live) -> int64_t {
     const int j = j0 + tok;
-    const bool live = j < context_len;
-    const int jc = live ? j : context_len - 1;  // dead lanes read a valid token and are masked
+    live = j < context_len;
+    const int jc = live ? j : context_len - 1;
     const int blk = jc / block_size;
     const int64_t page = min(max(table[blk], 0), num_blocks - 1);
-    // offset of (token, kv head g, d-chunk row 0, this lane's half)
-    const int64_t base = ((page * row_chunks + (int64_t)g * chunks) * block_size + (jc - blk * block_size)) * 16 + 8 * half;
-    const int64_t chunk_stride = (int64_t)block_size * 16;
-    f16x8 kv[CH];
+    return ((page * row_chunks + (int64_t)g * chunks) * block_size + (jc - blk * block_size)) * 16 + 8 * half;
+  };
+  // K of a block is fetched while the block before it is being worked on (the wave's own blocks are its only
+  // source of memory parallelism, one wave per SIMD at most): with the registers for it (head_dim <= 128) the
+  // loop holds K of the next block and V of this one in flight together.
+  constexpr bool kPrefetch = CH <= 8;
+  constexpr int kStep = kPaGenericWaves * 32;
+  f16x8 kk[CH], vv[kPrefetch ? CH : 1];
+  bool live_next = false;
+  int64_t base_next = 0;
+  if (wave * 32 < context_len) {
+    base_next = locate(wave * 32, live_next);
 #pragma unroll
     for (int c = 0; c < CH; ++c)
-      if (c < chunks) kv[c] = ld128_stream(key_cache + base + c * chunk_stride);
+      if (c < chunks) kk[c] = ld128_stream(key_cache + base_next + c * chunk_stride);
+  }
+  for (int j0 = wave * 32; j0 < context_len; j0 += kStep) {
+    const bool live = live_next;
+    const int64_t base = base_next;
     float part = 0.f;
 #pragma unroll
     for (int c = 0; c < CH; ++c)
       if (c < chunks) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) part += (float)qv[c][e] * (float)kv[c][e];
+        for (int e = 0; e < 8; ++e) part += (float)qv[c][e] * (float)kk[c][e];
       }
+    // V of this block; then, K of the wave's next block into the registers the scores have just freed
+    auto load_v = [&](auto& dst) {
 #pragma unroll
-    for (int c = 0; c < CH; ++c)
-      if (c < chunks) kv[c] = ld128_stream(value_cache + base + c * chunk_stride);
+      for (int c = 0; c < CH; ++c)
+        if (c < chunks) dst[c] = ld128_stream(value_cache + base + c * chunk_stride);
+    };
+    auto load_next_k = [&] {
+      if (j0 + kStep < context_len) {
+        base_next = locate(j0 + kStep, live_next);
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+          if (c < chunks) kk[c] = ld128_stream(key_cache + base_next + c * chunk_stride);
+      }
+    };
+    if constexpr (kPrefetch) {
+      load_v(vv);
+      load_next_k();
+    } else {
+      load_v(kk);
+    }
     part += __shfl_xor(part, 1);
     const float sc = live ? part * scale_log2 : -__builtin_inff();
     float mx = sc;
@@ -807,18 +841,26 @@ __global__ __launch_bounds__(kPaGenericWaves* kWave) void pa_decode_generic(
     const float p = live ? __builtin_amdgcn_exp2f(sc - m_new) : 0.f;
     m = m_new;
     l = l * alpha + p;
+    auto add_pv = [&](const auto& src) {
 #pragma unroll
-    for (int c = 0; c < CH; ++c)
-      if (c < chunks) {
+      for (int c = 0; c < CH; ++c)
+        if (c < chunks) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          // cache contents of dead tokens are arbitrary (possibly NaN): they must not reach the sum
-          const float v = live ? (float)kv[c][e] : 0.f;
-          acc[c][e] = acc[c][e] * alpha + p * v;
+          for (int e = 0; e < 8; ++e) {
+            // cache contents of dead tokens are arbitrary (possibly NaN): they must not reach the sum
+            const float v = live ? (float)src[c][e] : 0.f;
+            acc[c][e] = acc[c][e] * alpha + p * v;
+          }
         }
-      }
+    };
+    if constexpr (kPrefetch) {
+      add_pv(vv);
+    } else {
+      add_pv(kk);
+      load_next_k();
+    }
   }
-  // add up the 32 tokens of the wave (lanes with the same half), then the four waves
+  // add up the 32 tokens of the wave (lanes with the same half), then the waves
   __shared__ float sm_acc[kPaGenericWaves][kPaGenericMaxD];
   __shared__ float sm_m[kPaGenericWaves], sm_l[kPaGenericWaves];
 #pragma unroll
@@ -840,7 +882,9 @@ __global__ __launch_bounds__(kPaGenericWaves* kWave) void pa_decode_generic(
   }
   __syncthreads();
   for (int d = threadIdx.x; d < head_dim; d += kPaGenericWaves * kWave) {
-    const float mx = fmaxf(fmaxf(sm_m[0], sm_m[1]), fmaxf(sm_m[2], sm_m[3]));
+    float mx = sm_m[0];
+#pragma unroll
+    for (int w = 1; w < kPaGenericWaves; ++w) mx = fmaxf(mx, sm_m[w]);
     float lsum = 0.f, a = 0.f;
 #pragma unroll
     for (int w = 0; w < kPaGenericWaves; ++w) {
@@ -914,7 +958,8 @@ static int pa_run(const void* q, const void* key_cache, const void* value_cache,
     const int64_t grid = (total + kPaXcds - 1) / kPaXcds * kPaXcds;
     if (grid > 0x7fffffff) return AOPS_ERR_INVALID_ARGUMENT;
     auto kernel = head_dim <= 64 ? pa_decode_generic<4> : head_dim <= 128 ? pa_decode_generic<8> : pa_decode_generic<16>;
-    kernel<<<(unsigned)grid, kPaGenericWaves * kWave, 0, s>>>(qp, kc, vc, block_tables, context_lens, op, (int)bs,
+    const int waves = pa_generic_waves(head_dim <= 128 ? 8 : 16);
+    kernel<<<(unsigned)grid, waves * kWave, 0, s>>>(qp, kc, vc, block_tables, context_lens, op, (int)bs,
                                                              (int)num_heads, (int)num_kv_heads, (int)head_dim,
                                                              (int)block_size, (int)max_blocks_per_seq, scale_log2,
                                                              (int)num_blocks);
