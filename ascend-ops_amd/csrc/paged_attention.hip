@@ -957,8 +957,9 @@ static int pa_run(const void* q, const void* key_cache, const void* value_cache,
     const int64_t total = bs * num_heads;
     const int64_t grid = (total + kPaXcds - 1) / kPaXcds * kPaXcds;
     if (grid > 0x7fffffff) return AOPS_ERR_INVALID_ARGUMENT;
-    auto kernel = head_dim <= 64 ? pa_decode_generic<4> : head_dim <= 128 ? pa_decode_generic<8> : pa_decode_generic<16>;
-    const int waves = pa_generic_waves(head_dim <= 128 ? 8 : 16);
+    const int ch = head_dim <= 64 ? 4 : head_dim <= 128 ? 8 : 16;  // d-chunk rows the registers are sized for
+    auto kernel = ch == 4 ? pa_decode_generic<4> : ch == 8 ? pa_decode_generic<8> : pa_decode_generic<16>;
+    const int waves = pa_generic_waves(ch);
     kernel<<<(unsigned)grid, waves * kWave, 0, s>>>(qp, kc, vc, block_tables, context_lens, op, (int)bs,
                                                              (int)num_heads, (int)num_kv_heads, (int)head_dim,
                                                              (int)block_size, (int)max_blocks_per_seq, scale_log2,
