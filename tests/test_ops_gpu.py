@@ -336,6 +336,36 @@ def test_grouped_matmul_every_kernel(ops, dev, variant, rows, K, N, E, counts):
     assert torch.all(y[end:] == 5.0)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_grouped_matmul_persistent_kernel_random_shapes(ops, dev, seed):
+    """The persistent kernel (variant 6) on seeded random problems: group sizes from empty to several tiles (every
+    number of live row blocks of a tile occurs), one to many work items per workgroup, 4 to 12 k tiles, so that the
+    hand-over of the operand pipeline from one work item to the next is exercised in all its forms."""
+    import random
+    rnd = random.Random(100 + seed)
+    g = _gen(100 + seed)
+    E = rnd.choice([1, 3, 8, 33, 70])
+    K = 128 * rnd.randint(2, 6)
+    N = 64 * rnd.randint(1, 9)
+    rows = rnd.choice([31, 321, 700, 1500, 3000])
+    routed = rnd.choice([rows, rnd.randint(0, rows)])
+    if rnd.random() < 0.5:
+        ids = torch.randint(0, E, (routed,), generator=g)
+    else:  # skewed: a few large groups, many small or empty ones
+        ids = (torch.rand(routed, generator=g) ** 3 * E).long().clamp(0, E - 1)
+    gl = torch.bincount(ids, minlength=E).cumsum(0).to(torch.int64)
+    x = torch.randn(rows, K, generator=g).half()
+    w = (torch.randn(E, K, N, generator=g) / K ** 0.5).half()   # logical [E, K, N]
+    y = torch.full((rows, N), 5.0, dtype=H, device=dev)
+    xd, wd, gd = x.to(dev), w.transpose(1, 2).contiguous().to(dev), gl.to(dev)   # storage [E, N, K]
+    code = cabi.lib().aops_grouped_matmul_variant_f16(6, xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y.data_ptr(),
+                                                      rows, K, E, N, cabi.stream(dev))
+    assert code == 0
+    ref = R.grouped_matmul_ref(x, w, gl)
+    torch.testing.assert_close(y.cpu()[:routed].float(), ref[:routed].float(), **GMM_TOL)
+    assert torch.all(y[routed:] == 5.0)
+
+
 @pytest.mark.parametrize(
     "rows,K,N,E,counts",
     [
