@@ -37,6 +37,16 @@ int device_cu_count() {
   return v;
 }
 
+hipError_t allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = -1;
+  const bool tracked = dev >= 0 && dev < 64;
+  if (tracked && (done.load(std::memory_order_relaxed) >> dev & 1)) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && tracked) done.fetch_or(uint64_t(1) << dev, std::memory_order_relaxed);
+  return e;
+}
+
 }  // namespace aops
 
 extern "C" int aops_version(void) { return 200; }

@@ -2,6 +2,8 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <stdint.h>
 
 #include "aops.h"
@@ -90,5 +92,10 @@ int record_launch_status(hipError_t e);
 // device to ask).  The one source of the CU count for every launcher that sizes a grid or a
 // partition by it.
 int device_cu_count();
+
+// Raises the dynamic LDS limit of `kernel` to `bytes` on the current device, once per device (the attribute
+// belongs to the kernel as loaded on one device; `done` is the caller's record, one bit per device, and
+// races on it are benign: the call is idempotent).
+hipError_t allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done);
 
 }  // namespace aops

@@ -478,13 +478,9 @@ static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* grou
   grid = grid / kXcds * kXcds;
   if (grid < kXcds) grid = kXcds;
   auto kernel = grouped_matmul_persistent_kernel<MB, NB, WN, SWIGLU, GATHER>;
-  static bool attr_set = false;  // benign race: the call is idempotent
-  if (!attr_set) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e != hipSuccess) return record_launch_status(e);
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // per device
+  if (const hipError_t le = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLds, lds_allowed); le != hipSuccess)
+    return record_launch_status(le);
   kernel<<<(unsigned)grid, 2 * WN * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts,
                                                           n, row_idx, idx_div, (uint32_t)x_rows);
   return record_launch_status(hipGetLastError());

@@ -604,13 +604,9 @@ static int gmm_dma_launch(const f16* x, const f16* w, const int64_t* group_list,
   grid = (grid + kXcds - 1) / kXcds * kXcds;
   if (grid > 0x7fffffff) return AOPS_ERR_INVALID_ARGUMENT;
   auto kernel = grouped_matmul_dma_kernel<MB, NB, WN, false, NS>;
-  static bool attr_set = false;  // benign race: the call is idempotent
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e != hipSuccess) return record_launch_status(e);
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // per device
+  if (const hipError_t le = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLds, lds_allowed); le != hipSuccess)
+    return record_launch_status(le);
   kernel<<<(unsigned)grid, 2 * WN * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts,
                                                           n, nullptr, 1);
   return record_launch_status(hipGetLastError());
@@ -756,13 +752,9 @@ static int launch_splitk(const f16* x, const f16* w, const int64_t* group_list, 
   static_assert(kStageBytes <= 160 * 1024, "LDS budget");
   auto kernel = grouped_matmul_dma_kernel<MB, NB, WN, true>;
   auto reduce = matmul_splitk_reduce<MB, NB, WN>;
-  static bool attr_set = false;  // benign race: the calls are idempotent
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kStageBytes);
-    if (e != hipSuccess) return record_launch_status(e);
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // per device
+  if (const hipError_t le = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kStageBytes, lds_allowed); le != hipSuccess)
+    return record_launch_status(le);
   kernel<<<(unsigned)(tiles * splits), 2 * WN * kWave, kStageBytes, stream>>>(x, w, nullptr, y, m, k, 1, n,
                                                                             workspace, splits);
   hipError_t e = hipGetLastError();
@@ -799,13 +791,9 @@ static int gmm_launch(const f16* x, const f16* w, const int64_t* group_list, f16
   grid = (grid + kXcds - 1) / kXcds * kXcds;
   if (grid > 0x7fffffff) return AOPS_ERR_INVALID_ARGUMENT;
   auto kernel = grouped_matmul_kernel<MB, NB, D, SWIGLU, GATHER>;
-  static bool attr_set = false;  // benign race: the call is idempotent
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e != hipSuccess) return record_launch_status(e);
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // per device
+  if (const hipError_t le = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLds, lds_allowed); le != hipSuccess)
+    return record_launch_status(le);
   kernel<<<(unsigned)grid, 4 * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts, n, row_idx,
                                                        idx_div, (uint32_t)x_rows);
   return record_launch_status(hipGetLastError());

@@ -110,13 +110,9 @@ int matmul_fewrows_launch(const f16* x, const f16* w, const int64_t* group_list,
                           int n, hipStream_t stream) {
   constexpr int kLds = kFrWaves * 2 * kFrPiece * (int)sizeof(f16) + kFrWaves * 16 * 17 * (int)sizeof(float);
   static_assert(kLds <= 160 * 1024, "LDS budget");
-  static bool attr_set = false;  // benign race: the call is idempotent
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(matmul_fewrows_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-    if (e != hipSuccess) return record_launch_status(e);
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // per device
+  if (const hipError_t le = allow_dynamic_lds(reinterpret_cast<const void*>(matmul_fewrows_kernel), kLds, lds_allowed); le != hipSuccess)
+    return record_launch_status(le);
   matmul_fewrows_kernel<<<(unsigned)(n / 16), kFrWaves * kWave, kLds, stream>>>(x, w, group_list, y, (int)m, k, n);
   return record_launch_status(hipGetLastError());
 }
