@@ -446,7 +446,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
             asm volatile("" ::: "memory");
             const int m = 32 * wm + 64 * i + u * kRowsPerUnit + r_r;
             if (m < tile_rows)
-              st128(y + (int64_t)(cur.row_begin + m) * n_out + col_w + q_r * 8, v);
+              st128_stream(y + (int64_t)(cur.row_begin + m) * n_out + col_w + q_r * 8, v);
           }
         }
       }
