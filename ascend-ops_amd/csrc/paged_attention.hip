@@ -8,8 +8,8 @@
 // read on the device only, so the grid is sized for the longest possible context and
 // workgroups past the end of their sequence exit at once.
 //
-// Main kernel (head_dim 64, 128 or 256; described for 128), one step = 32 tokens of one kv head =
-// 8 KiB of K + 8 KiB of V:
+// Main kernel (every head_dim that is a multiple of 16 up to 256 with pages of a multiple of 16 tokens;
+// described for 128), one step = 32 tokens of one kv head = 8 KiB of K + 8 KiB of V:
 //  * For one kv head a page holds K as [8 d-chunks][block_size tokens][16 halfs].  A lane
 //    (n = lane%16, kg = lane/16) loads, for token n of a 16-token group, the 16 bytes that hold
 //    d = 32s + 8kg ..+7 (s = 0..3).  That register IS the per-lane operand of
@@ -48,11 +48,12 @@ struct PaChunking {
 };
 
 constexpr int kPaUnit = kPaWaves * kPaStep;  // 256 tokens: one step of every wave
-constexpr int kPaMaxGroup = 16;              // query heads per kv head the matrix-core kernel serves
+constexpr int kPaMaxGroup = 16;              // query heads of a sub-group: one per lane of a row of the score product
 constexpr int kPaXcds = 8;                   // workgroup i runs on XCD i % 8
 
-// Batches of up to kPaPlanMax sequences can use the balanced partition; above 64 sequences it is
-// computed by a one-workgroup kernel into kPaPlanInts(bs) ints behind the partial results.
+// Batches of up to kPaPlanMax sequences can use the balanced partition; above 64 sequences every workgroup
+// of the balanced kernel computes it in LDS and one of them leaves it, for the merge kernel, in the ints
+// behind the partial results.
 constexpr int64_t kPaPlanMax = 4096;
 constexpr int64_t kPaMaxChunks = 512;  // partial results per (sequence, head) at most
 constexpr int64_t kPaMaxShares = 256;
@@ -95,25 +96,45 @@ static PaChunking pa_chunking(int64_t bs, int64_t num_kv_heads, int64_t block_si
   return c;
 }
 
+// How a head of D elements is cut up for the matrix core: kFull slices of 32 d, plus, when D is an odd
+// multiple of 16, a last slice that holds 16 d in the lanes kg < 2 and zeros in the lanes kg >= 2.
+template <int D>
+struct PaDims {
+  static_assert(D % 16 == 0 && D >= 16 && D <= 256, "head_dim: a multiple of 16 up to 256");
+  static constexpr int kFull = D / 32;
+  static constexpr int kTail = (D % 32) / 16;
+  static constexpr int kSlices = kFull + kTail;
+  static constexpr int kOutBlocks = D / 16;  // blocks of 16 d of O^T
+};
+
 // Per-lane slice of a 32-token tile: [token group][s] holds X[token 16t + n][d = 32s + 8kg ..+7],
-// s = 0 .. NS-1 with NS = head_dim / 32.
+// s = 0 .. NS-1 with NS = PaDims<D>::kSlices.
 template <int NS>
 using PaRegs = f16x8[2][NS];
 
-template <int NS>
+// tail_live: this lane holds data of the half slice (kg < 2); the other lanes must not load (their
+// address lies past the head's last d-chunk row) and hold zeros.
+template <int D>
 __device__ __forceinline__ void pa_issue_loads(const f16* __restrict__ cache, int64_t off0, int64_t off1,
-                                               uint32_t lane_off, uint32_t s_stride, PaRegs<NS>& r) {
+                                               uint32_t lane_off, uint32_t s_stride, bool tail_live,
+                                               PaRegs<PaDims<D>::kSlices>& r) {
+  constexpr int kFull = PaDims<D>::kFull;
 #pragma unroll
   for (int g = 0; g < 2; ++g) {
     const f16* base = cache + (g == 0 ? off0 : off1) + lane_off;  // token group g of the step
 #pragma unroll
-    for (int s = 0; s < NS; ++s) r[g][s] = ld128_stream(base + s * s_stride);
+    for (int s = 0; s < kFull; ++s) r[g][s] = ld128_stream(base + s * s_stride);
+    if constexpr (PaDims<D>::kTail) {
+      f16x8 t = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (tail_live) t = ld128_stream(base + kFull * s_stride);
+      r[g][kFull] = t;
+    }
   }
 }
 
-template <int NS>
+template <int D>
 struct PaState {
-  f32x4 o[2 * NS];  // O^T blocks: lane (head n, kg), o[db][i] <-> d = 16 db + 4 kg + i
+  f32x4 o[PaDims<D>::kOutBlocks];  // O^T blocks: lane (head n, kg), o[db][i] <-> d = 16 db + 4 kg + i
   float m;     // running maximum of head n (identical in the four lanes of a head)
   float l;     // this lane's share of the running sum
 };
@@ -121,7 +142,7 @@ struct PaState {
 // S^T[token][head] = K . Q^T, scaled to log2 units; lane (head n, kg) gets tokens
 // 16*(e/4) + 4kg + e%4, e = 0..7, of the step.
 // QLDS: the Q^T fragments are read from LDS (q_lds = this lane's slice, fragment s 512 halfs further)
-// instead of being held in registers: at head_dim 256 they would push the kernel into scratch.
+// instead of being held in registers: where many of them are needed they would push the kernel into scratch.
 template <int NS, bool QLDS>
 __device__ __forceinline__ void pa_scores(const PaRegs<NS>& k, const f16x8 (&qreg)[QLDS ? 1 : NS],
                                           const f16* q_lds, float scale_log2, float (&sc)[8]) {
@@ -160,8 +181,8 @@ __device__ __forceinline__ void pa_scores(const PaRegs<NS>& k, const f16x8 (&qre
 }
 
 // Online softmax update; returns the P^T operand (lane (head n, kg), element e <-> token e).
-template <int NS>
-__device__ __forceinline__ f16x8 pa_softmax(float (&sc)[8], PaState<NS>& st) {
+template <int D>
+__device__ __forceinline__ f16x8 pa_softmax(float (&sc)[8], PaState<D>& st) {
   float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
                    fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
   mx = fmaxf(mx, __shfl_xor(mx, 16));
@@ -179,22 +200,23 @@ __device__ __forceinline__ f16x8 pa_softmax(float (&sc)[8], PaState<NS>& st) {
   st.l = st.l * alpha + psum;
   if (__builtin_amdgcn_ballot_w64(alpha != 1.0f)) {  // the maximum rarely moves after the start
 #pragma unroll
-    for (int db = 0; db < 2 * NS; ++db)
+    for (int db = 0; db < PaDims<D>::kOutBlocks; ++db)
 #pragma unroll
       for (int i = 0; i < 4; ++i) st.o[db][i] *= alpha;
   }
   return pt;
 }
 
-// O^T += V^T . P^T with V transposed on the matrix core.
-template <int NS>
-__device__ __forceinline__ void pa_accumulate(const PaRegs<NS>& v, const f16x8 (&sel)[2], f16x8 pt,
-                                              PaState<NS>& st) {
+// O^T += V^T . P^T with V transposed on the matrix core; the transposed tile serves every sub-group of
+// query heads.
+template <int D, int NSUB>
+__device__ __forceinline__ void pa_accumulate(const PaRegs<PaDims<D>::kSlices>& v, const f16x8 (&sel)[2],
+                                              const f16x8 (&pt)[NSUB], PaState<D> (&st)[NSUB]) {
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int s = 0; s < NS; ++s) {
+  for (int s = 0; s < PaDims<D>::kSlices; ++s) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < (s < PaDims<D>::kFull ? 2 : 1); ++u) {  // the half slice has d = 32s + n only
       // [token][d = 32s + 16u + n]: lane (n, kg) receives tokens 4kg..4kg+3 of each group
       const f32x4 x0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(v[0][s], sel[u], zero4, 0, 0, 0);
       const f32x4 x1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(v[1][s], sel[u], zero4, 0, 0, 0);
@@ -204,53 +226,92 @@ __device__ __forceinline__ void pa_accumulate(const PaRegs<NS>& v, const f16x8 (
         vt[i] = (f16)x0[i];
         vt[4 + i] = (f16)x1[i];
       }
-      st.o[2 * s + u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt, pt, st.o[2 * s + u], 0, 0, 0);
+#pragma unroll
+      for (int sg = 0; sg < NSUB; ++sg)
+        st[sg].o[2 * s + u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vt, pt[sg], st[sg].o[2 * s + u], 0, 0, 0);
     }
   }
 }
 
+// LDS of the main kernels (dynamic): [Q^T fragments, where they are kept there][acc: kPaWaves x hp x D floats]
+// [m: kPaWaves x hp][l: kPaWaves x hp]; hp = query heads per pass of the cross-wave merge (chosen by the host so
+// that the whole fits 64 KiB).
+template <int D, int NSUB>
+constexpr bool pa_q_in_lds() { return PaDims<D>::kSlices * NSUB > 4; }
+template <int D, int NSUB>
+constexpr int pa_q_lds_halfs() { return pa_q_in_lds<D, NSUB>() ? NSUB * PaDims<D>::kSlices * kWave * 8 : 0; }
+
+// What a workgroup needs to know about the launch besides its chunk.
+struct PaGeom {
+  int num_heads, num_kv_heads, block_size, max_blocks_per_seq, max_splits, num_blocks;
+  int group;        // query heads per kv head
+  int wg_heads;     // query heads per workgroup (16 * NSUB at most); a kv head with more is served by several
+  int virt;         // workgroups per kv head: ceil(group / wg_heads)
+  int merge_heads;  // hp above
+  float scale_log2;
+};
+
 // One chunk of one (sequence b, kv head g): tokens chunk_start .. chunk_start + chunk_len - 1, the
-// steps dealt round robin to the eight waves, which are merged through LDS at the end.  `group` =
-// query heads per kv head, GMAX = the power of two it is rounded up to (<= 16; sizes the LDS
-// arrays).  FINAL: the chunk is the whole sequence, so the normalised output is written directly;
-// otherwise the partial result goes to slot `split` of the (sequence, head)'s max_splits slots.
+// steps dealt round robin to the eight waves, which are merged through LDS at the end.  The workgroup
+// serves the nh query heads head0 .. head0 + nh - 1 of the kv head in NSUB sub-groups of 16 (a lane of the
+// score product holds one head of a sub-group); K and V of a step are loaded once and V is transposed
+// once for all sub-groups.  final: the chunk is the whole sequence, so the normalised output is written
+// directly; otherwise the partial result goes to slot `split` of the (sequence, head)'s max_splits slots.
 // Called by all threads of the workgroup with uniform arguments.
-template <int D, int GMAX, bool FINAL>
+template <int D, int NSUB>
 __device__ __forceinline__ void pa_process_chunk(
     const f16* __restrict__ q, const f16* __restrict__ key_cache,
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
-    float* __restrict__ part_o, float* __restrict__ part_ml, f16* __restrict__ out, int b, int g,
-    int context_len, int chunk_start, int chunk_len, int split, int num_kv_heads, int block_size,
-    int max_blocks_per_seq, int max_splits, float scale_log2, int num_blocks, int group) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, f16* __restrict__ out, bool final, int b, int g,
+    int head0, int nh, int context_len, int chunk_start, int chunk_len, int split, const PaGeom& ge) {
   constexpr int kPaD = D;
-  constexpr int NS = D / 32;
+  constexpr int NS = PaDims<D>::kSlices;
+  constexpr int kFull = PaDims<D>::kFull;
+  constexpr int NOB = PaDims<D>::kOutBlocks;
   const int nsteps = (chunk_len + kPaStep - 1) / kPaStep;
+  const int block_size = ge.block_size;
+  const int max_blocks_per_seq = ge.max_blocks_per_seq;
 
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int lane = threadIdx.x & (kWave - 1);
   const int n = lane & 15;
   const int kg = lane >> 4;
-  const int num_heads = num_kv_heads * group;
+  const bool tail_live = kg < 2;
+  const int num_heads = ge.num_heads;
 
-  // Q^T operand: lane (head n, kg) holds q[head n][32s + 8kg ..+7]; heads >= group are zero rows.
-  constexpr bool QLDS = NS > 4;
-  f16x8 qreg[QLDS ? 1 : NS];
-  __shared__ __attribute__((aligned(16))) f16 sm_q[QLDS ? NS * kWave * 8 : 8];
+  extern __shared__ __attribute__((aligned(16))) unsigned char pa_lds[];
+  f16* sm_q = reinterpret_cast<f16*>(pa_lds);
+  float* sm_acc = reinterpret_cast<float*>(pa_lds + pa_q_lds_halfs<D, NSUB>() * sizeof(f16));
+  const int hp = ge.merge_heads;
+  float* sm_m = sm_acc + kPaWaves * hp * kPaD;
+  float* sm_l = sm_m + kPaWaves * hp;
+
+  // Q^T operand: lane (head n of a sub-group, kg) holds q[head][32s + 8kg ..+7]; heads >= nh are zero
+  // rows, and so are d >= D in the half slice.
+  constexpr bool QLDS = pa_q_in_lds<D, NSUB>();
+  f16x8 qreg[QLDS ? 1 : NSUB][QLDS ? 1 : NS];
   const f16* q_lds = sm_q + lane * 8;
   {
     const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    const f16* qp = q + ((int64_t)b * num_heads + g * group + (n < group ? n : 0)) * kPaD + 8 * kg;
-    if constexpr (QLDS) {  // every wave uses the same fragments: wave 0 fetches them
-      if (wave == 0) {
+    if (!QLDS || wave == 0) {  // in LDS every wave uses the same fragments: wave 0 fetches them
 #pragma unroll
-        for (int s = 0; s < NS; ++s)
-          *reinterpret_cast<f16x8*>(sm_q + (s * kWave + lane) * 8) = n < group ? ld128(qp + 32 * s) : zero8;
+      for (int sg = 0; sg < NSUB; ++sg) {
+        const int hl = 16 * sg + n;
+        const bool head_live = hl < nh;
+        const f16* qp = q + ((int64_t)b * num_heads + head0 + (head_live ? hl : 0)) * kPaD + 8 * kg;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+          f16x8 frag = zero8;
+          if (head_live && (s < kFull || tail_live)) frag = ld128(qp + 32 * s);
+          if constexpr (QLDS) {
+            *reinterpret_cast<f16x8*>(sm_q + ((sg * NS + s) * kWave + lane) * 8) = frag;
+          } else {
+            qreg[sg][s] = frag;
+          }
+        }
       }
-      __syncthreads();
-    } else {
-#pragma unroll
-      for (int s = 0; s < NS; ++s) qreg[s] = n < group ? ld128(qp + 32 * s) : zero8;
     }
+    if constexpr (QLDS) __syncthreads();
   }
   // Selector operands of the transposing product: sel[u][k][n] = (k == n + 16u), k = 8kg + e.
   f16x8 sel[2];
@@ -259,20 +320,24 @@ __device__ __forceinline__ void pa_process_chunk(
 #pragma unroll
     for (int e = 0; e < 8; ++e) sel[u][e] = (8 * kg + e == n + 16 * u) ? (f16)1.0f : (f16)0.0f;
 
-  PaState<NS> st;
+  PaState<D> st[NSUB];
 #pragma unroll
-  for (int db = 0; db < 2 * NS; ++db) st.o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
-  st.m = kNegBig;
-  st.l = 0.f;
+  for (int sg = 0; sg < NSUB; ++sg) {
+#pragma unroll
+    for (int db = 0; db < NOB; ++db) st[sg].o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    st[sg].m = kNegBig;
+    st[sg].l = 0.f;
+  }
 
   // Element offsets inside one page for this lane: d-chunk rows are block_size*16 halfs apart
   // (this lane starts in row kg/2), the two halves of a granule 8 halfs, tokens 16 halfs.
   const uint32_t lane_off = (uint32_t)(kg >> 1) * (uint32_t)block_size * 16u +
                             (uint32_t)(kg & 1) * 8u + (uint32_t)n * 16u;
   const uint32_t s_stride = 2u * (uint32_t)block_size * 16u;  // 32 d further = two d-chunk rows
-  const int64_t page_elems = (int64_t)num_kv_heads * kPaD * block_size;
+  const int64_t page_elems = (int64_t)ge.num_kv_heads * kPaD * block_size;
   const int64_t head_off = (int64_t)g * kPaD * block_size;
   const int32_t* table = block_tables + (int64_t)b * max_blocks_per_seq;
+  const int num_blocks = ge.num_blocks;
 
   // Offset of the 16-token group `grp` of a step (wave uniform).  Page sizes are multiples of 16, so a
   // group never straddles two pages; the two groups of a step may (page sizes that are odd multiples).
@@ -292,9 +357,11 @@ __device__ __forceinline__ void pa_process_chunk(
     const int64_t next_off0 = has_next ? page_offset(next, 0) : 0;
     const int64_t next_off1 = has_next ? page_offset(next, 1) : 0;
     const int step_token0 = chunk_start + step * kPaStep;
-    float sc[8];
-    pa_scores<NS, QLDS>(kreg, qreg, q_lds, scale_log2, sc);
-    if (has_next) pa_issue_loads(key_cache, next_off0, next_off1, lane_off, s_stride, kreg);
+    float sc[NSUB][8];
+#pragma unroll
+    for (int sg = 0; sg < NSUB; ++sg)
+      pa_scores<NS, QLDS>(kreg, qreg[QLDS ? 0 : sg], q_lds + sg * (NS * kWave * 8), ge.scale_log2, sc[sg]);
+    if (has_next) pa_issue_loads<D>(key_cache, next_off0, next_off1, lane_off, s_stride, tail_live, kreg);
     if (step_token0 + kPaStep > context_len) {  // wave uniform: last, partial step of the sequence
       // Cache contents past the end of the sequence are arbitrary (possibly NaN): drop their
       // scores and zero their V rows before they reach the matrix core.
@@ -303,22 +370,27 @@ __device__ __forceinline__ void pa_process_chunk(
       for (int g = 0; g < 2; ++g) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (step_token0 + 16 * g + 4 * kg + i >= context_len) sc[4 * g + i] = -__builtin_inff();
+          if (step_token0 + 16 * g + 4 * kg + i >= context_len) {
+#pragma unroll
+            for (int sg = 0; sg < NSUB; ++sg) sc[sg][4 * g + i] = -__builtin_inff();
+          }
         if (step_token0 + 16 * g + n >= context_len) {
 #pragma unroll
           for (int s = 0; s < NS; ++s) vreg[g][s] = zero8;
         }
       }
     }
-    const f16x8 pt = pa_softmax(sc, st);
-    pa_accumulate(vreg, sel, pt, st);
-    if (has_next) pa_issue_loads(value_cache, next_off0, next_off1, lane_off, s_stride, vreg);
+    f16x8 pt[NSUB];
+#pragma unroll
+    for (int sg = 0; sg < NSUB; ++sg) pt[sg] = pa_softmax<D>(sc[sg], st[sg]);
+    pa_accumulate<D, NSUB>(vreg, sel, pt, st);
+    if (has_next) pa_issue_loads<D>(value_cache, next_off0, next_off1, lane_off, s_stride, tail_live, vreg);
   };
   auto first_loads = [&](PaRegs<NS>& kreg, PaRegs<NS>& vreg, int step) {
     if (step < nsteps) {
       const int64_t off0 = page_offset(step, 0), off1 = page_offset(step, 1);
-      pa_issue_loads(key_cache, off0, off1, lane_off, s_stride, kreg);
-      pa_issue_loads(value_cache, off0, off1, lane_off, s_stride, vreg);
+      pa_issue_loads<D>(key_cache, off0, off1, lane_off, s_stride, tail_live, kreg);
+      pa_issue_loads<D>(value_cache, off0, off1, lane_off, s_stride, tail_live, vreg);
     }
   };
   // (A second register set, with the step after next in flight as well, was tried up to head_dim
@@ -327,47 +399,54 @@ __device__ __forceinline__ void pa_process_chunk(
   first_loads(kreg, vreg, wave);
   for (int step = wave; step < nsteps; step += kPaWaves) do_step(kreg, vreg, step, kPaWaves);
 
-  // The four lanes of a head hold disjoint shares of the sum.
-  float l_head = st.l;
-  l_head += __shfl_xor(l_head, 16);
-  l_head += __shfl_xor(l_head, 32);
-
-  // Merge the waves of the workgroup through LDS and emit one partial per query head.
-  __shared__ float sm_acc[kPaWaves][GMAX][kPaD];
-  __shared__ float sm_m[kPaWaves][GMAX];
-  __shared__ float sm_l[kPaWaves][GMAX];
-  if (n < group) {
+  // Merge the waves of the workgroup through LDS and emit one result per query head, hp heads of one
+  // sub-group per pass.
 #pragma unroll
-    for (int db = 0; db < 2 * NS; ++db)
-      *reinterpret_cast<f32x4*>(&sm_acc[wave][n][16 * db + 4 * kg]) = st.o[db];
-    if (kg == 0) {
-      sm_m[wave][n] = st.m;
-      sm_l[wave][n] = l_head;
-    }
-  }
-  __syncthreads();
-  for (int e = threadIdx.x; e < group * kPaD; e += kPaWaves * kWave) {
-    const int h = e / kPaD;
-    const int d = e - h * kPaD;
-    float mx = sm_m[0][h];
+  for (int sg = 0; sg < NSUB; ++sg) {
+    // The four lanes of a head hold disjoint shares of the sum.
+    float l_head = st[sg].l;
+    l_head += __shfl_xor(l_head, 16);
+    l_head += __shfl_xor(l_head, 32);
+    const int sub_end = min(nh, 16 * sg + 16);
+    for (int h0 = 16 * sg; h0 < sub_end; h0 += hp) {
+      const int cnt = min(hp, sub_end - h0);
+      const int r = 16 * sg + n - h0;  // this lane's head inside the pass
+      if (r >= 0 && r < cnt) {
+        float* dst = sm_acc + ((int64_t)(wave * hp + r)) * kPaD + 4 * kg;
 #pragma unroll
-    for (int w = 1; w < kPaWaves; ++w) mx = fmaxf(mx, sm_m[w][h]);
-    float lsum = 0.f, a = 0.f;
-#pragma unroll
-    for (int w = 0; w < kPaWaves; ++w) {
-      const float wt = __builtin_amdgcn_exp2f(sm_m[w][h] - mx);
-      lsum += sm_l[w][h] * wt;
-      a += sm_acc[w][h][d] * wt;
-    }
-    if (FINAL) {
-      out[((int64_t)b * num_heads + g * group + h) * kPaD + d] = (f16)(lsum > 0.f ? a / lsum : 0.f);
-    } else {
-      const int64_t slot = ((int64_t)b * num_heads + g * group + h) * max_splits + split;
-      part_o[slot * kPaD + d] = a;
-      if (d == 0) {
-        part_ml[slot * 2 + 0] = mx;
-        part_ml[slot * 2 + 1] = lsum;
+        for (int db = 0; db < NOB; ++db) *reinterpret_cast<f32x4*>(dst + 16 * db) = st[sg].o[db];
+        if (kg == 0) {
+          sm_m[wave * hp + r] = st[sg].m;
+          sm_l[wave * hp + r] = l_head;
+        }
       }
+      __syncthreads();
+      for (int e = threadIdx.x; e < cnt * kPaD; e += kPaWaves * kWave) {
+        const int h = e / kPaD;
+        const int d = e - h * kPaD;
+        float mx = sm_m[h];
+#pragma unroll
+        for (int w = 1; w < kPaWaves; ++w) mx = fmaxf(mx, sm_m[w * hp + h]);
+        float lsum = 0.f, a = 0.f;
+#pragma unroll
+        for (int w = 0; w < kPaWaves; ++w) {
+          const float wt = __builtin_amdgcn_exp2f(sm_m[w * hp + h] - mx);
+          lsum += sm_l[w * hp + h] * wt;
+          a += sm_acc[(w * hp + h) * kPaD + d] * wt;
+        }
+        const int64_t head = (int64_t)b * num_heads + head0 + h0 + h;
+        if (final) {
+          out[head * kPaD + d] = (f16)(lsum > 0.f ? a / lsum : 0.f);
+        } else {
+          const int64_t slot = head * ge.max_splits + split;
+          part_o[slot * kPaD + d] = a;
+          if (d == 0) {
+            part_ml[slot * 2 + 0] = mx;
+            part_ml[slot * 2 + 1] = lsum;
+          }
+        }
+      }
+      if (h0 + hp < sub_end || sg + 1 < NSUB) __syncthreads();  // the next pass reuses the arrays
     }
   }
 }
@@ -391,17 +470,20 @@ __global__ __launch_bounds__(kPaRankMax) void pa_rank_sequences(const int32_t* _
   order[rank] = t;
 }
 
-// grid = (max_splits, Hkv, bs), block = 8 waves: one chunk of chunk_tokens tokens per workgroup.
-template <int D, int GMAX, bool FINAL>
+// grid = (max_splits, Hkv * virt, bs), block = 8 waves: one chunk of chunk_tokens tokens per workgroup.  A
+// sequence that fits one chunk gets its output written directly; the others leave partial results.
+template <int D, int NSUB>
 __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
     const f16* __restrict__ q, const f16* __restrict__ key_cache,
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ context_lens, float* __restrict__ part_o,
-    float* __restrict__ part_ml, f16* __restrict__ out, int num_kv_heads, int block_size, int max_blocks_per_seq,
-    int chunk_tokens, int max_splits, float scale_log2, int num_blocks, int group,
+    float* __restrict__ part_ml, f16* __restrict__ out, const PaGeom ge, int chunk_tokens,
     const int32_t* __restrict__ order) {
   const int split = blockIdx.x;
-  const int g = blockIdx.y;
+  const int g = (int)blockIdx.y / ge.virt;
+  const int v = (int)blockIdx.y - g * ge.virt;
+  const int head0 = g * ge.group + v * ge.wg_heads;
+  const int nh = min(ge.wg_heads, ge.group - v * ge.wg_heads);
   // Workgroups are handed out in index order, so they take the sequences longest first: with
   // one resident workgroup per CU the short sequences then fill the gaps the long ones leave
   // (longest-processing-time-first).  For batches of up to 64 sequences every wave finds the
@@ -420,19 +502,18 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_partial(
     if (hit) b = __builtin_ctzll(hit);  // exactly one lane has each rank
   }
   // a length beyond the block table would walk off the table row
-  const int context_len = min(context_lens[b], max_blocks_per_seq * block_size);
+  const int context_len = min(context_lens[b], ge.max_blocks_per_seq * ge.block_size);
   const int chunk_start = split * chunk_tokens;
   if (chunk_start >= context_len) {
-    if (FINAL) {  // empty sequence: zeros
-      for (int e = threadIdx.x; e < group * D; e += kPaWaves * kWave)
-        out[((int64_t)b * num_kv_heads * group + g * group) * D + e] = (f16)0.f;
+    if (split == 0) {  // empty sequence: zeros
+      for (int e = threadIdx.x; e < nh * D; e += kPaWaves * kWave)
+        out[((int64_t)b * ge.num_heads + head0) * D + e] = (f16)0.f;
     }
     return;
   }
-  pa_process_chunk<D, GMAX, FINAL>(q, key_cache, value_cache, block_tables, part_o, part_ml, out, b, g,
-                                   context_len, chunk_start, min(context_len - chunk_start, chunk_tokens),
-                                   split, num_kv_heads, block_size, max_blocks_per_seq, max_splits,
-                                   scale_log2, num_blocks, group);
+  pa_process_chunk<D, NSUB>(q, key_cache, value_cache, block_tables, part_o, part_ml, out,
+                            context_len <= chunk_tokens, b, g, head0, nh, context_len, chunk_start,
+                            min(context_len - chunk_start, chunk_tokens), split, ge);
 }
 
 // Balanced partition for batches of up to 64 sequences.  Lane l of every wave holds sequence l:
@@ -465,91 +546,117 @@ __device__ __forceinline__ int pa_share_of(int x, int wgs, int total) {
   return (int)((((int64_t)x + 1) * wgs - 1) / total);
 }
 
-// The same partition for batches of more than 64 sequences, computed once by one workgroup into
-//   plan[0] = total units, plan[1 + b] = units in front of sequence b, plan[1 + bs + b] = its clamped
-//   length, plan[1 + 2*bs + w] = the sequence that holds the first unit of share w.
-constexpr int kPaPlanThreads = 1024;
+// The same partition for batches of 65 .. kPaPlanMax sequences: every workgroup of the balanced kernel
+// scans the lengths itself (thread t holds kPaPlanPer consecutive sequences) and keeps, in LDS behind the
+// merge arrays, lds_plan[b] = units in front of sequence b and lds_plan[bs + b] = its clamped length,
+// then [2*bs] = total units, [2*bs + 1] = the sequence that holds the share's first unit.  Workgroup
+// (0, 0) also writes   plan[0] = total, plan[1 + b] = units in front of b, plan[1 + bs + b] = its length
+// to global memory for the merge kernel.
+constexpr int kPaPlanPer = (int)(kPaPlanMax / (kPaWaves * kWave));  // 8 sequences per thread
+static_assert(kPaPlanPer * kPaWaves * kWave == kPaPlanMax, "every sequence has a thread");
 
-__global__ __launch_bounds__(kPaPlanThreads) void pa_plan_kernel(const int32_t* __restrict__ context_lens,
-                                                                 int bs, int max_len, int wgs_max,
-                                                                 int32_t* __restrict__ plan) {
-  __shared__ int wave_sum[kPaPlanThreads / kWave];
-  __shared__ int carry_s;
+__device__ __forceinline__ void pa_block_plan(const int32_t* __restrict__ context_lens, int bs, int max_len,
+                                              int wgs_max, int w, int* __restrict__ lds_plan,
+                                              int32_t* __restrict__ plan, bool publish) {
   const int t = threadIdx.x;
   const int lane = t & (kWave - 1);
   const int wave = t / kWave;
-  if (t == 0) carry_s = 0;
-  __syncthreads();
-  for (int b0 = 0; b0 < bs; b0 += kPaPlanThreads) {
-    const int b = b0 + t;
-    const int len = b < bs ? min(max(context_lens[b], 0), max_len) : 0;
-    const int units = (len + kPaUnit - 1) / kPaUnit;
-    int incl = units;
+  const int per = (bs + kPaWaves * kWave - 1) / (kPaWaves * kWave);  // <= kPaPlanPer
+  int len[kPaPlanPer], units[kPaPlanPer];
+  int mine = 0;
 #pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-      const int up = __shfl_up(incl, d);
-      if (lane >= d) incl += up;
-    }
-    if (lane == kWave - 1) wave_sum[wave] = incl;
-    __syncthreads();
-    int before = carry_s + incl - units;
-    for (int v = 0; v < wave; ++v) before += wave_sum[v];
-    if (b < bs) {
-      plan[1 + b] = before;
-      plan[1 + bs + b] = len;
-    }
-    __syncthreads();
-    if (t == kPaPlanThreads - 1) carry_s = before + units;
-    __syncthreads();
+  for (int i = 0; i < kPaPlanPer; ++i) {
+    const int b = t * per + i;
+    len[i] = (i < per && b < bs) ? min(max(context_lens[b], 0), max_len) : 0;
+    units[i] = (len[i] + kPaUnit - 1) / kPaUnit;
+    mine += units[i];
   }
-  const int total = carry_s;
-  if (t == 0) plan[0] = total;
-  if (total == 0) return;
-  // every sequence names itself as the start of the shares whose first unit it holds
+  int incl = mine;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int up = __shfl_up(incl, d);
+    if (lane >= d) incl += up;
+  }
+  int* wave_sum = lds_plan + 2 * bs + 2;  // kPaWaves ints
+  if (lane == kWave - 1) wave_sum[wave] = incl;
+  __syncthreads();
+  int before = incl - mine;
+  int total = 0;
+#pragma unroll
+  for (int v = 0; v < kPaWaves; ++v) {
+    const int ws = wave_sum[v];
+    if (v < wave) before += ws;
+    total += ws;
+  }
   const int wgs = min(wgs_max, total);
-  for (int b = t; b < bs; b += kPaPlanThreads) {
-    const int before = plan[1 + b];  // written by this thread
-    const int units = (plan[1 + bs + b] + kPaUnit - 1) / kPaUnit;
-    if (units == 0) continue;
-    // shares w with before <= floor(w * total / wgs) < before + units
-    int w = (int)(((int64_t)before * wgs + total - 1) / total);
-    for (; w < wgs && (int)((int64_t)w * total / wgs) < before + units; ++w) plan[1 + 2 * bs + w] = b;
+  const int lo = (total > 0 && w < wgs) ? (int)((int64_t)w * total / wgs) : -1;
+  if (t == 0) {
+    lds_plan[2 * bs] = total;
+    lds_plan[2 * bs + 1] = bs;  // stays if the share is empty
+    if (publish) plan[0] = total;
   }
+  __syncthreads();  // [2*bs + 1] is initialised before the one thread below overwrites it
+#pragma unroll
+  for (int i = 0; i < kPaPlanPer; ++i) {
+    const int b = t * per + i;
+    if (i < per && b < bs) {
+      lds_plan[b] = before;
+      lds_plan[bs + b] = len[i];
+      if (publish) {
+        plan[1 + b] = before;
+        plan[1 + bs + b] = len[i];
+      }
+      if (units[i] > 0 && before <= lo && lo < before + units[i]) lds_plan[2 * bs + 1] = b;
+    }
+    before += units[i];
+  }
+  __syncthreads();
 }
 
-// grid = (wgs, Hkv), block = 8 waves.  Workgroup w walks through its share of the batch's units,
-// sequence by sequence; the part of sequence b it covers becomes partial result number
-// w - (share holding b's first unit) of that sequence.  plan == nullptr: at most 64 sequences, the
-// partition is computed by every wave (pa_units); otherwise it is read from pa_plan_kernel's output.
-template <int D, int GMAX>
+// ints of LDS the plan above needs
+static inline size_t pa_block_plan_ints(int64_t bs) { return bs > kWave ? (size_t)(2 * bs + 2 + kPaWaves) : 0; }
+
+// grid = (wgs, Hkv * virt), block = 8 waves.  Workgroup w walks through its share of the batch's units,
+// sequence by sequence; a sequence that lies inside one share gets its output written directly, otherwise
+// the part of sequence b the share covers becomes partial result number w - (share holding b's first unit)
+// of that sequence.  Up to 64 sequences the partition is computed by every wave (pa_units); above that by
+// the workgroup (pa_block_plan).
+template <int D, int NSUB>
 __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_balanced(
     const f16* __restrict__ q, const f16* __restrict__ key_cache,
     const f16* __restrict__ value_cache, const int32_t* __restrict__ block_tables,
     const int32_t* __restrict__ context_lens, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int bs, int num_kv_heads, int block_size, int max_blocks_per_seq,
-    int max_splits, float scale_log2, int num_blocks, int group, const int32_t* __restrict__ plan) {
+    float* __restrict__ part_ml, f16* __restrict__ out, int bs, const PaGeom ge, int32_t* __restrict__ plan) {
   const int w = blockIdx.x;
-  const int g = blockIdx.y;
-  if (plan) {
-    const int total = plan[0];
+  const int g = (int)blockIdx.y / ge.virt;
+  const int v = (int)blockIdx.y - g * ge.virt;
+  const int head0 = g * ge.group + v * ge.wg_heads;
+  const int nh = min(ge.wg_heads, ge.group - v * ge.wg_heads);
+  const int max_len = ge.max_blocks_per_seq * ge.block_size;
+  if (bs > kWave) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char pa_lds[];
+    int* lds_plan = reinterpret_cast<int*>(pa_lds + pa_q_lds_halfs<D, NSUB>() * sizeof(f16)) +
+                    kPaWaves * ge.merge_heads * (D + 2);
+    pa_block_plan(context_lens, bs, max_len, (int)gridDim.x, w, lds_plan, plan, w == 0 && blockIdx.y == 0);
+    const int total = lds_plan[2 * bs];
     const int wgs = min((int)gridDim.x, total);
     if (w >= wgs) return;
     const int lo = (int)((int64_t)w * total / wgs);
     const int hi = (int)((int64_t)(w + 1) * total / wgs);
     int cur = lo;
-    int b = plan[1 + 2 * bs + w];
+    int b = lds_plan[2 * bs + 1];
     while (cur < hi && b < bs) {
-      const int before = plan[1 + b];
-      const int len = plan[1 + bs + b];
+      const int before = lds_plan[b];
+      const int len = lds_plan[bs + b];
       const int units = (len + kPaUnit - 1) / kPaUnit;
       if (units > 0) {
         const int seg_end = min(hi, before + units);
         const int tok0 = (cur - before) * kPaUnit;
         const int tok1 = min((seg_end - before) * kPaUnit, len);
-        const int slot = w - pa_share_of(before, wgs, total);
-        pa_process_chunk<D, GMAX, false>(q, key_cache, value_cache, block_tables, part_o, part_ml, nullptr, b, g,
-                                         len, tok0, tok1 - tok0, slot, num_kv_heads, block_size,
-                                         max_blocks_per_seq, max_splits, scale_log2, num_blocks, group);
+        const int first = pa_share_of(before, wgs, total);
+        const bool whole = pa_share_of(before + units - 1, wgs, total) == first;
+        pa_process_chunk<D, NSUB>(q, key_cache, value_cache, block_tables, part_o, part_ml, out, whole, b, g,
+                                  head0, nh, len, tok0, tok1 - tok0, w - first, ge);
         cur = seg_end;
         if (cur < hi) __syncthreads();  // the LDS arrays of the chunk are reused
       }
@@ -557,7 +664,7 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_balanced(
     }
     return;
   }
-  const PaUnits pu = pa_units(context_lens, bs, max_blocks_per_seq * block_size);
+  const PaUnits pu = pa_units(context_lens, bs, max_len);
   // no more shares than units: every share then holds at least one unit, and the shares of a
   // sequence are consecutive
   const int wgs = min((int)gridDim.x, pu.total);
@@ -576,38 +683,39 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_balanced(
     const int seg_end = min(hi, before + units);
     const int tok0 = (cur - before) * kPaUnit;
     const int tok1 = min((seg_end - before) * kPaUnit, len);
-    const int slot = w - pa_share_of(before, wgs, pu.total);
-    pa_process_chunk<D, GMAX, false>(q, key_cache, value_cache, block_tables, part_o, part_ml, nullptr, b, g,
-                                     len, tok0, tok1 - tok0, slot, num_kv_heads, block_size,
-                                     max_blocks_per_seq, max_splits, scale_log2, num_blocks, group);
+    const int first = pa_share_of(before, wgs, pu.total);
+    const bool whole = pa_share_of(before + units - 1, wgs, pu.total) == first;
+    pa_process_chunk<D, NSUB>(q, key_cache, value_cache, block_tables, part_o, part_ml, out, whole, b, g,
+                              head0, nh, len, tok0, tok1 - tok0, w - first, ge);
     cur = seg_end;
     if (cur < hi) __syncthreads();  // the LDS arrays of the chunk are reused
   }
 }
 
-// grid = (Hq, bs), block = 4 waves.  Every wave works out the weights 2^(m_s - max m) of the partial
+// grid = (Hq, bs), block = 4 waves.  Sequences whose output the attention kernel has written itself (one
+// partial result) are left alone.  Every wave works out the weights 2^(m_s - max m) of the partial
 // results (a lane per result); wave v then adds up the results s = v, v+4, ... with eight row loads in
-// flight (a lane holds head_dim/64 neighbouring output elements), and the four sums meet in LDS.
+// flight (a lane holds kPer neighbouring output elements: 1, 2 or 4 for head_dim up to 64, 128, 256), and
+// the four sums meet in LDS.
 constexpr int kPaMergeWaves = 4;
 constexpr int kPaMergeMaxSplits = (int)kPaMaxChunks;  // weights kept in LDS; pa_chunking never cuts a sequence finer
 
-template <int kPaD>
+template <int kPer>
 __global__ __launch_bounds__(kPaMergeWaves* kWave) void pa_decode_merge(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
-    const int32_t* __restrict__ context_lens, f16* __restrict__ o, int num_heads, int chunk_tokens,
+    const int32_t* __restrict__ context_lens, f16* __restrict__ o, int head_dim, int num_heads, int chunk_tokens,
     int max_splits, int balanced_wgs, int bs, int max_len, const int32_t* __restrict__ plan) {
-  constexpr int kPer = kPaD / kWave;  // output elements per lane
   typedef float fvec __attribute__((ext_vector_type(kPer)));
   __shared__ float wts[kPaMergeMaxSplits];
-  __shared__ float red[kPaMergeWaves][kPaD];
+  __shared__ float red[kPaMergeWaves][kPer * kWave];
   const int h = blockIdx.x;
   const int b = blockIdx.y;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   const int context_len = context_lens[b];
-  const int64_t out = ((int64_t)b * num_heads + h) * kPaD;
+  const int64_t out = ((int64_t)b * num_heads + h) * head_dim;
   if (context_len <= 0) {
-    if (threadIdx.x < kPaD) o[out + threadIdx.x] = (f16)0.f;
+    if ((int)threadIdx.x < head_dim) o[out + threadIdx.x] = (f16)0.f;
     return;
   }
   int nsplit;
@@ -624,10 +732,12 @@ __global__ __launch_bounds__(kPaMergeWaves* kWave) void pa_decode_merge(
     const int wgs = min(balanced_wgs, pu.total);
     nsplit = pa_share_of(before + units - 1, wgs, pu.total) - pa_share_of(before, wgs, pu.total) + 1;
   } else {
-    nsplit = (context_len + chunk_tokens - 1) / chunk_tokens;
+    nsplit = (min(context_len, max_len) + chunk_tokens - 1) / chunk_tokens;
   }
+  if (nsplit <= 1) return;  // the attention kernel wrote this sequence's output itself
   nsplit = min(nsplit, min(max_splits, kPaMergeMaxSplits));
   const int64_t base = ((int64_t)b * num_heads + h) * max_splits;
+  const bool act = lane * kPer < head_dim;  // lanes past the end of the head hold nothing
 
   // weights: the same in every wave; wave 0 leaves them in LDS
   constexpr int kMlPerLane = kPaMergeMaxSplits / kWave;
@@ -669,7 +779,8 @@ __global__ __launch_bounds__(kPaMergeWaves* kWave) void pa_decode_merge(
     for (int j = 0; j < kInFlight; ++j) {
       const int s = s0 + j * kPaMergeWaves;
       const int sc = min(s, nsplit - 1);  // past the end: a valid row with weight 0
-      v[j] = *reinterpret_cast<const fvec*>(&part_o[(base + sc) * kPaD + lane * kPer]);
+      v[j] = acc;                         // any finite value for the idle lanes
+      if (act) v[j] = *reinterpret_cast<const fvec*>(&part_o[(base + sc) * head_dim + lane * kPer]);
       wt[j] = s < nsplit ? wts[sc] : 0.f;
     }
 #pragma unroll
@@ -680,7 +791,7 @@ __global__ __launch_bounds__(kPaMergeWaves* kWave) void pa_decode_merge(
 #pragma unroll
   for (int e = 0; e < kPer; ++e) red[wave][lane * kPer + e] = acc[e];
   __syncthreads();
-  if (threadIdx.x < kPaD) {
+  if ((int)threadIdx.x < head_dim) {
     float a = 0.f;
 #pragma unroll
     for (int v = 0; v < kPaMergeWaves; ++v) a += red[v][threadIdx.x];
@@ -688,46 +799,77 @@ __global__ __launch_bounds__(kPaMergeWaves* kWave) void pa_decode_merge(
   }
 }
 
-template <int kPaD, int GMAX>
-static void pa_launch(const f16* q, const f16* kc, const f16* vc, const int32_t* bt,
-                      const int32_t* cl, f16* o, float* part_o, float* part_ml, int bs,
-                      int num_heads, int num_kv_heads, int block_size, int max_blocks_per_seq,
-                      PaChunking ch, hipStream_t s, int num_blocks, int32_t* order) {
-  const float scale_log2 = kLog2e / __builtin_sqrtf((float)kPaD);
-  if (ch.balanced_wgs > 0) {
-    const int32_t* plan = nullptr;
-    if (bs > kWave) {  // `order` is the int area behind the partial results
-      pa_plan_kernel<<<1, kPaPlanThreads, 0, s>>>(cl, bs, max_blocks_per_seq * block_size, ch.balanced_wgs, order);
-      plan = order;
-    }
-    dim3 bgrid((unsigned)ch.balanced_wgs, (unsigned)num_kv_heads);
-    pa_decode_balanced<kPaD, GMAX><<<bgrid, kPaWaves * kWave, 0, s>>>(
-        q, kc, vc, bt, cl, part_o, part_ml, bs, num_kv_heads, block_size, max_blocks_per_seq,
-        ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads, plan);
-    dim3 mgrid((unsigned)num_heads, (unsigned)bs);
-    pa_decode_merge<kPaD><<<mgrid, kPaMergeWaves * kWave, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
-                                           ch.max_splits, ch.balanced_wgs, bs,
-                                           max_blocks_per_seq * block_size, plan);
-    return;
-  }
-  dim3 grid((unsigned)ch.max_splits, (unsigned)num_kv_heads, (unsigned)bs);
-  if (bs <= kWave || bs > kPaRankMax) order = nullptr;  // ranked inside the kernel / not ranked at all
-  if (order) pa_rank_sequences<<<1, kPaRankMax, 0, s>>>(cl, bs, order);
-  if (ch.max_splits == 1) {
-    pa_decode_partial<kPaD, GMAX, true><<<grid, kPaWaves * kWave, 0, s>>>(
-        q, kc, vc, bt, cl, part_o, part_ml, o, num_kv_heads, block_size, max_blocks_per_seq,
-        ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads, order);
-    return;
-  }
-  pa_decode_partial<kPaD, GMAX, false><<<grid, kPaWaves * kWave, 0, s>>>(
-      q, kc, vc, bt, cl, part_o, part_ml, o, num_kv_heads, block_size, max_blocks_per_seq,
-      ch.chunk_tokens, ch.max_splits, scale_log2, num_blocks, num_heads / num_kv_heads, order);
-  dim3 mgrid((unsigned)num_heads, (unsigned)bs);
-  pa_decode_merge<kPaD><<<mgrid, kPaMergeWaves * kWave, 0, s>>>(part_o, part_ml, cl, o, num_heads, ch.chunk_tokens,
-                                         ch.max_splits, 0, bs, max_blocks_per_seq * block_size, nullptr);
+// Arguments of a launch of the main kernels.
+struct PaCall {
+  const f16 *q, *kc, *vc;
+  const int32_t *bt, *cl;
+  f16* o;
+  float *part_o, *part_ml;
+  int32_t* ints;  // int area behind the partial results: length order or plan
+  int bs, head_dim;
+  PaGeom ge;
+  PaChunking ch;
+  hipStream_t s;
+};
+
+// Query-head sub-groups of 16 a workgroup serves: K and V stay in registers across them, so their number is
+// bounded by the registers the accumulators of a sub-group take.
+static int pa_subgroups(int64_t head_dim, int64_t group) {
+  const int64_t fit = head_dim <= 128 ? 2 : 1;
+  const int64_t want = (group + kPaMaxGroup - 1) / kPaMaxGroup;
+  return (int)(want < fit ? want : fit);
 }
 
-// Generic path for every other shape (head_dim a multiple of 16 up to 256, any block size, any
+static size_t pa_lds_bytes(int q_halfs, int merge_heads, int head_dim, int64_t bs, bool balanced) {
+  return (size_t)q_halfs * sizeof(f16) + (size_t)kPaWaves * merge_heads * (head_dim + 2) * sizeof(float) +
+         (balanced ? pa_block_plan_ints(bs) * sizeof(int) : 0);
+}
+
+// Heads per pass of the cross-wave merge: as many of a sub-group's as keep the workgroup's LDS within 64 KiB,
+// in passes of equal size.
+static int pa_merge_heads(int q_halfs, int head_dim, int heads, int64_t bs, bool balanced) {
+  const int sub = heads < kPaMaxGroup ? heads : kPaMaxGroup;
+  const int64_t budget = 64 * 1024 - (int64_t)q_halfs * (int64_t)sizeof(f16) -
+                         (int64_t)(balanced ? pa_block_plan_ints(bs) * sizeof(int) : 0);
+  int64_t cap = budget / (int64_t)(kPaWaves * (head_dim + 2) * sizeof(float));
+  if (cap < 1) cap = 1;
+  if (cap > sub) cap = sub;
+  const int passes = (int)((sub + cap - 1) / cap);
+  return (sub + passes - 1) / passes;
+}
+
+template <int D, int NSUB>
+static void pa_launch(PaCall c) {
+  constexpr int kQHalfs = pa_q_lds_halfs<D, NSUB>();
+  const bool balanced = c.ch.balanced_wgs > 0;
+  c.ge.merge_heads = pa_merge_heads(kQHalfs, D, c.ge.wg_heads < c.ge.group ? c.ge.wg_heads : c.ge.group, c.bs, balanced);
+  const size_t lds = pa_lds_bytes(kQHalfs, c.ge.merge_heads, D, c.bs, balanced);
+  const unsigned kv_wgs = (unsigned)(c.ge.num_kv_heads * c.ge.virt);
+  const int max_len = c.ge.max_blocks_per_seq * c.ge.block_size;
+  auto merge = [&](const int32_t* plan) {
+    dim3 mgrid((unsigned)c.ge.num_heads, (unsigned)c.bs);
+    auto kernel = D <= 64 ? pa_decode_merge<1> : D <= 128 ? pa_decode_merge<2> : pa_decode_merge<4>;
+    kernel<<<mgrid, kPaMergeWaves * kWave, 0, c.s>>>(c.part_o, c.part_ml, c.cl, c.o, D, c.ge.num_heads,
+                                                     c.ch.chunk_tokens, c.ch.max_splits, c.ch.balanced_wgs, c.bs,
+                                                     max_len, plan);
+  };
+  if (balanced) {
+    int32_t* plan = c.bs > kWave ? c.ints : nullptr;
+    dim3 bgrid((unsigned)c.ch.balanced_wgs, kv_wgs);
+    pa_decode_balanced<D, NSUB><<<bgrid, kPaWaves * kWave, lds, c.s>>>(c.q, c.kc, c.vc, c.bt, c.cl, c.part_o,
+                                                                        c.part_ml, c.o, c.bs, c.ge, plan);
+    merge(plan);
+    return;
+  }
+  dim3 grid((unsigned)c.ch.max_splits, kv_wgs, (unsigned)c.bs);
+  int32_t* order = (c.bs <= kWave || c.bs > kPaRankMax) ? nullptr : c.ints;  // ranked inside the kernel / not at all
+  if (order) pa_rank_sequences<<<1, kPaRankMax, 0, c.s>>>(c.cl, c.bs, order);
+  pa_decode_partial<D, NSUB><<<grid, kPaWaves * kWave, lds, c.s>>>(c.q, c.kc, c.vc, c.bt, c.cl, c.part_o, c.part_ml,
+                                                                   c.o, c.ge, c.ch.chunk_tokens, order);
+  if (c.ch.max_splits > 1) merge(nullptr);
+}
+
+// Generic path for page sizes that are not a multiple of 16 tokens (head_dim a multiple of 16 up to 256, any
 // whole number of query heads per kv head): one workgroup of eight waves per (sequence, query head).
 // A wave takes every eighth block of 32 tokens; lane (token = lane / 2, half = lane % 2) loads, d-chunk
 // row by d-chunk row, the 16 bytes that hold d = 16c + 8*half ..+7 of its token, so that a load
@@ -906,14 +1048,15 @@ static bool pa_args_valid(int64_t bs, int64_t num_heads, int64_t num_kv_heads, i
   return true;
 }
 
-// Shapes served by the MFMA kernel; everything else that is valid takes the generic kernel.
-static bool pa_fast_shape(int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
-                          int64_t block_size) {
-  if ((head_dim != 64 && head_dim != 128 && head_dim != 256) || block_size % 16 != 0) return false;
-  // a lane of the score product holds one of at most 16 query heads of the kv head, and the cross-wave
-  // merge keeps 8 x group x head_dim floats in LDS (at most 66 KB): up to 16 heads, 8 at head_dim 256
-  const int64_t group = num_heads / num_kv_heads;
-  return group <= kPaMaxGroup && group * head_dim <= kPaMaxGroup * 128;
+// Shapes served by the matrix-core kernels: every head_dim the operator admits, any number of query heads
+// per kv head, pages of a multiple of 16 tokens (a 16-token group of a step never straddles two pages).
+// Other page sizes take the generic kernel.
+static bool pa_fast_shape(int64_t block_size) { return block_size % 16 == 0; }
+
+// Workgroups per kv head (a workgroup serves at most 16 * pa_subgroups query heads of it).
+static int64_t pa_virtual_heads(int64_t head_dim, int64_t group) {
+  const int64_t per_wg = (int64_t)kPaMaxGroup * pa_subgroups(head_dim, group);
+  return (group + per_wg - 1) / per_wg;
 }
 
 }  // namespace aops
@@ -924,8 +1067,9 @@ extern "C" size_t aops_paged_attention_workspace(int64_t bs, int64_t num_heads,
   using namespace aops;
   if (!pa_args_valid(bs, num_heads, num_kv_heads, head_dim, block_size, max_blocks_per_seq))
     return 0;
-  if (!pa_fast_shape(num_heads, num_kv_heads, head_dim, block_size)) return 16;  // not used
-  const PaChunking ch = pa_chunking(bs, num_kv_heads, block_size, max_blocks_per_seq);
+  if (!pa_fast_shape(block_size)) return 16;  // not used
+  const PaChunking ch = pa_chunking(bs, num_kv_heads * pa_virtual_heads(head_dim, num_heads / num_kv_heads),
+                                    block_size, max_blocks_per_seq);
   // partial results, then the ints of the length order or of the balanced partition's plan
   return (size_t)bs * (size_t)num_heads * (size_t)ch.max_splits * (size_t)(head_dim + 2) * sizeof(float) +
          pa_tail_ints(bs) * sizeof(int32_t);
@@ -952,7 +1096,7 @@ static int pa_run(const void* q, const void* key_cache, const void* value_cache,
   const f16* kc = static_cast<const f16*>(key_cache);
   const f16* vc = static_cast<const f16*>(value_cache);
   f16* op = static_cast<f16*>(o);
-  if (!pa_fast_shape(num_heads, num_kv_heads, head_dim, block_size)) {
+  if (!pa_fast_shape(block_size)) {
     const float scale_log2 = kLog2e / __builtin_sqrtf((float)head_dim);
     const int64_t total = bs * num_heads;
     const int64_t grid = (total + kPaXcds - 1) / kPaXcds * kPaXcds;
@@ -969,35 +1113,65 @@ static int pa_run(const void* q, const void* key_cache, const void* value_cache,
   const size_t need = aops_paged_attention_workspace(bs, num_heads, num_kv_heads, head_dim,
                                                      block_size, max_blocks_per_seq);
   if (!workspace || workspace_bytes < need) return AOPS_ERR_WORKSPACE;
-  const PaChunking ch = pa_chunking(bs, num_kv_heads, block_size, max_blocks_per_seq);
-  float* part_o = static_cast<float*>(workspace);
-  float* part_ml = part_o + (size_t)bs * num_heads * ch.max_splits * head_dim;
-  int32_t* order = reinterpret_cast<int32_t*>(part_ml + (size_t)bs * num_heads * ch.max_splits * 2);
-#define AOPS_PA_CASE(D, G)                                                                      \
-  case G:                                                                                       \
-    pa_launch<D, G>(qp, kc, vc, block_tables, context_lens, op, part_o, part_ml, (int)bs,       \
-                    (int)num_heads, (int)num_kv_heads, (int)block_size, (int)max_blocks_per_seq, \
-                    ch, s, (int)num_blocks, order);                                             \
-    break;
-#define AOPS_PA_GROUPS(D)     \
-  switch (gmax) {             \
-    AOPS_PA_CASE(D, 1)        \
-    AOPS_PA_CASE(D, 2)        \
-    AOPS_PA_CASE(D, 4)        \
-    AOPS_PA_CASE(D, 8)        \
-    AOPS_PA_CASE(D, 16)       \
-  }
   const int64_t group = num_heads / num_kv_heads;
-  if (group > kPaMaxGroup) return AOPS_ERR_INVALID_ARGUMENT;  // pa_fast_shape admits no such shape
-  const int gmax = group <= 1 ? 1 : group <= 2 ? 2 : group <= 4 ? 4 : group <= 8 ? 8 : 16;
-  if (head_dim == 64) {
-    AOPS_PA_GROUPS(64)
-  } else if (head_dim == 128) {
-    AOPS_PA_GROUPS(128)
-  } else {
-    AOPS_PA_GROUPS(256)
+  const int nsub = pa_subgroups(head_dim, group);
+  const int64_t virt = pa_virtual_heads(head_dim, group);
+  if (num_kv_heads * virt > 65535) return AOPS_ERR_INVALID_ARGUMENT;  // grid dimension
+  PaCall c;
+  c.ch = pa_chunking(bs, num_kv_heads * virt, block_size, max_blocks_per_seq);
+  c.q = qp;
+  c.kc = kc;
+  c.vc = vc;
+  c.bt = block_tables;
+  c.cl = context_lens;
+  c.o = op;
+  c.part_o = static_cast<float*>(workspace);
+  c.part_ml = c.part_o + (size_t)bs * num_heads * c.ch.max_splits * head_dim;
+  c.ints = reinterpret_cast<int32_t*>(c.part_ml + (size_t)bs * num_heads * c.ch.max_splits * 2);
+  c.bs = (int)bs;
+  c.head_dim = (int)head_dim;
+  c.s = s;
+  c.ge.num_heads = (int)num_heads;
+  c.ge.num_kv_heads = (int)num_kv_heads;
+  c.ge.block_size = (int)block_size;
+  c.ge.max_blocks_per_seq = (int)max_blocks_per_seq;
+  c.ge.max_splits = c.ch.max_splits;
+  c.ge.num_blocks = (int)num_blocks;
+  c.ge.group = (int)group;
+  c.ge.wg_heads = kPaMaxGroup * nsub;
+  c.ge.virt = (int)virt;
+  c.ge.merge_heads = 0;  // set by pa_launch
+  c.ge.scale_log2 = kLog2e / __builtin_sqrtf((float)head_dim);
+#define AOPS_PA_CASE(D)                      \
+  case D / 16:                               \
+    if constexpr (D <= 128) {                \
+      if (nsub == 2) {                       \
+        pa_launch<D, 2>(c);                  \
+        break;                               \
+      }                                      \
+    }                                        \
+    pa_launch<D, 1>(c);                      \
+    break;
+  switch (head_dim / 16) {
+    AOPS_PA_CASE(16)
+    AOPS_PA_CASE(32)
+    AOPS_PA_CASE(48)
+    AOPS_PA_CASE(64)
+    AOPS_PA_CASE(80)
+    AOPS_PA_CASE(96)
+    AOPS_PA_CASE(112)
+    AOPS_PA_CASE(128)
+    AOPS_PA_CASE(144)
+    AOPS_PA_CASE(160)
+    AOPS_PA_CASE(176)
+    AOPS_PA_CASE(192)
+    AOPS_PA_CASE(208)
+    AOPS_PA_CASE(224)
+    AOPS_PA_CASE(240)
+    AOPS_PA_CASE(256)
+    default:
+      return AOPS_ERR_INVALID_ARGUMENT;  // pa_args_valid admits no other head_dim
   }
-#undef AOPS_PA_GROUPS
 #undef AOPS_PA_CASE
   return record_launch_status(hipGetLastError());
 }

@@ -268,9 +268,9 @@ int aops_moe_combine_f16(const void* y, const int32_t* inverse_idx, const float*
  * The kernels split every sequence into fixed-size chunks of the KV cache and keep partial
  * results in `workspace`; aops_paged_attention_workspace() returns the bytes needed (the
  * counterpart of the reference's GetWorkspaceSize phase; 0 = shape not supported).  head_dim must
- * be a multiple of 16 up to 256.  head_dim 64, 128 or 256 with block_size a multiple of 16 and
- * up to 16 query heads per kv head (8 at head_dim 256) runs on the matrix cores; every other
- * shape takes a generic, untuned kernel.  A sequence with context_len <= 0 gets zeros; a context_len beyond
+ * be a multiple of 16 up to 256; any whole number of query heads per kv head.  With block_size a
+ * multiple of 16 the operator runs on the matrix cores; other page sizes take a generic, slower
+ * kernel.  A sequence with context_len <= 0 gets zeros; a context_len beyond
  * max_blocks_per_seq*block_size is cut there.  Block-table entries outside [0, num_blocks) are
  * clamped into it (garbage in, garbage out, no fault).
  * Replaces aclnnPagedAttentionExGetWorkspaceSize + aclnnPagedAttentionEx

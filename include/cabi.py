@@ -1,12 +1,13 @@
-"""Test helper: libaops.so loaded through ctypes, with the argument types of every function taken from the
-declarations in include/aops.h.  The GPU parity tests call the C ABI through this (raw device pointers,
-sizes, stream handle), exactly as a native caller would; the product itself binds the library from C++."""
+"""ctypes view of the C ABI for tools that sit outside the product (the parity tests, bench.py): libaops.so with
+the argument types of every function taken from the declarations in aops.h, which lies next to this file.  They
+call the C ABI through this (raw device pointers, sizes, stream handle), exactly as a native caller would; the
+product itself binds the library from C++."""
 import ctypes
 import os
 import re
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "aops.h")
+HEADER = os.path.join(os.path.dirname(os.path.abspath(__file__)), "aops.h")
 LIBRARY = os.path.join(ROOT, "ascend-ops_amd", "ascend910a_extras", "libaops.so")
 
 _SCALARS = {

@@ -4,7 +4,7 @@ import sys
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-for p in (ROOT, os.path.join(ROOT, "ascend-ops_amd"), os.path.join(ROOT, "tests")):
+for p in (ROOT, os.path.join(ROOT, "ascend-ops_amd"), os.path.join(ROOT, "tests"), os.path.join(ROOT, "include")):
     if p not in sys.path:
         sys.path.insert(0, p)
 

@@ -688,9 +688,9 @@ def test_paged_attention_batch_larger_than_a_wave(ops, dev, B, Hq, Hkv, P):
         (2, 6, 2, 128, 128, [130, 700]),        # 3 query heads per kv head
         (2, 4, 4, 256, 32, [33, 0]),            # head_dim 256, one empty sequence
         (2, 32, 2, 128, 64, [100, 1000]),       # 16 query heads per kv head (matrix-core path)
-        (2, 8, 2, 128, 24, [25, 300]),          # block size not a multiple of 32
-        (1, 5, 5, 48, 8, [77]),                 # head_dim 48
-        (2, 32, 1, 64, 16, [70, 300]),          # more than 16 query heads per kv head: generic kernel
+        (2, 8, 2, 128, 24, [25, 300]),          # block size not a multiple of 16: generic kernel
+        (1, 5, 5, 48, 8, [77]),                 # head_dim 48 on 8-token pages: generic kernel
+        (2, 32, 1, 64, 16, [70, 300]),          # more than 16 query heads per kv head
         (2, 24, 1, 64, 32, [33, 129]),
         (3, 17, 1, 64, 16, [1, 16, 250]),
         (2, 40, 2, 128, 16, [100, 37]),         # 20 heads per kv head at head_dim 128
@@ -786,14 +786,72 @@ def test_paged_attention_balanced_partition(ops, dev, B, Hq, Hkv, P, maxlen, see
     assert torch.equal(_run_pa(ops, dev, case), o)
 
 
-def test_paged_attention_wide_groups_take_the_generic_kernel():
-    """The matrix-core kernel holds one of at most 16 query heads of a kv head per lane (8 at head_dim 256);
-    wider groups must be routed to the generic kernel, which needs no workspace (the query answers 16)."""
+def test_paged_attention_only_odd_page_sizes_take_the_generic_kernel():
+    """Every head size and every number of query heads per kv head runs on the matrix cores as long as the page size
+    is a multiple of 16 tokens; the generic kernel, which needs no workspace (the query answers 16), is left with the
+    other page sizes."""
     ws = cabi.lib().aops_paged_attention_workspace
-    for hq, hkv, d in [(32, 1, 64), (24, 1, 64), (17, 1, 64), (40, 2, 128), (9, 1, 256)]:
-        assert ws(2, hq, hkv, d, 16, 64) == 16
-    for hq, hkv, d in [(16, 1, 64), (32, 2, 128), (8, 1, 256)]:
+    for hq, hkv, d in [(32, 1, 64), (24, 1, 64), (17, 1, 64), (40, 2, 128), (9, 1, 256), (80, 1, 128), (4, 4, 48),
+                       (16, 4, 96), (8, 2, 160), (8, 8, 16), (6, 2, 240)]:
         assert ws(2, hq, hkv, d, 16, 64) > 16
+    for p in (8, 24, 100):
+        assert ws(2, 32, 8, 128, p, 64) == 16
+
+
+@pytest.mark.parametrize("D", [16, 32, 48, 80, 96, 112, 144, 160, 176, 192, 208, 224, 240])
+@pytest.mark.parametrize(
+    "B,Hq,Hkv,P,lens",
+    [
+        (3, 8, 2, 16, [1, 50, 700]),            # whole sequences per workgroup or few chunks
+        (2, 6, 2, 128, [3000, 257]),            # balanced partition, sequences cut into partial results
+        (70, 4, 4, 32, None),                   # more sequences than lanes
+    ],
+)
+def test_paged_attention_every_head_size(ops, dev, D, B, Hq, Hkv, P, lens):
+    """Head sizes that are a multiple of 16 but not 64, 128 or 256: whole slices of 32 elements plus, for odd multiples
+    of 16, a half slice whose upper lanes hold zeros.  Unused cache slots hold NaN and unused table entries -1."""
+    if lens is None:
+        rnd = torch.Generator().manual_seed(D)
+        lens = torch.randint(0, 400, (B,), generator=rnd).tolist()
+        lens[7] = 1500
+    assert cabi.lib().aops_paged_attention_workspace(B, Hq, Hkv, D, P, 64) > 16   # not the generic kernel
+    case = _paged_case(B, Hq, Hkv, D, P, lens, seed=D + B, poison=True)
+    o = _run_pa(ops, dev, case)
+    ref = R.paged_attention_ref(*case)
+    assert o.shape == (B, Hq, D) and not torch.isnan(o).any()
+    torch.testing.assert_close(o.float(), ref.float(), **TOL)
+    assert (o.float() - ref.float()).abs().max() < 3e-3
+
+
+@pytest.mark.parametrize(
+    "B,Hq,Hkv,D,P,lens",
+    [
+        (2, 17, 1, 64, 16, [1, 250]),           # 17 heads per kv head: two sub-groups, the second with one head
+        (2, 24, 1, 128, 32, [33, 1290]),        # 24
+        (3, 64, 2, 128, 128, [130, 5000, 0]),   # 32: two full sub-groups per workgroup; balanced partition
+        (2, 40, 1, 64, 16, [70, 300]),          # 40: two workgroups per kv head (32 + 8 heads)
+        (2, 80, 2, 96, 48, [100, 1000]),        # 40 at head_dim 96
+        (2, 20, 1, 256, 64, [64, 65]),          # above head_dim 128 a workgroup serves 16 heads: 16 + 4
+        (2, 36, 2, 192, 16, [700, 3]),          # 18 at head_dim 192
+        (2, 16, 1, 256, 32, [33, 700]),         # 16 heads at head_dim 256: the cross-wave merge runs in passes
+        (70, 48, 2, 128, 16, None),             # 24 heads per kv head, more sequences than lanes
+    ],
+)
+def test_paged_attention_wide_groups(ops, dev, B, Hq, Hkv, D, P, lens):
+    """More than 16 query heads per kv head: a workgroup serves up to two sub-groups of 16 heads from one set of K/V
+    registers (head_dim up to 128), and kv heads with more query heads than that are shared by several workgroups."""
+    if lens is None:
+        rnd = torch.Generator().manual_seed(5)
+        lens = torch.randint(0, 300, (B,), generator=rnd).tolist()
+        lens[11] = 2000
+    assert cabi.lib().aops_paged_attention_workspace(B, Hq, Hkv, D, P, 128) > 16
+    case = _paged_case(B, Hq, Hkv, D, P, lens, seed=17, poison=True)
+    o = _run_pa(ops, dev, case)
+    ref = R.paged_attention_ref(*case)
+    assert o.shape == (B, Hq, D) and not torch.isnan(o).any()
+    torch.testing.assert_close(o.float(), ref.float(), **TOL)
+    assert (o.float() - ref.float()).abs().max() < 3e-3
+    assert torch.equal(_run_pa(ops, dev, case), o)
 
 
 def test_paged_attention_very_long_context(ops, dev):
