@@ -20,18 +20,24 @@ int device_cu_count() {
   constexpr int kMaxDevices = 64;
   constexpr int kDefault = 256;
   static std::atomic<int> cus[kMaxDevices];  // 0 = not asked yet; every writer stores the same value
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) {
-    (void)hipGetLastError();  // no device: not an error of the caller's launch
+  // "No device to ask" (a workspace query on a machine without a GPU) answers with an MI355X's count; any
+  // other failure of the runtime is kept for aops_last_hip_error() instead of being swallowed.
+  auto fallback = [](hipError_t e) {
+    (void)hipGetLastError();
+    if (e != hipErrorNoDevice && e != hipErrorInvalidDevice && e != hipErrorInsufficientDriver &&
+        e != hipErrorNotInitialized)
+      (void)record_launch_status(e);
     return kDefault;
-  }
+  };
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fallback(e);
   if (dev < 0 || dev >= kMaxDevices) return kDefault;
   int v = cus[dev].load(std::memory_order_relaxed);
   if (v == 0) {
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) {
-      (void)hipGetLastError();
-      v = kDefault;
-    }
+    e = hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return fallback(e);
+    if (v <= 0) v = kDefault;
     cus[dev].store(v, std::memory_order_relaxed);
   }
   return v;

@@ -226,7 +226,10 @@ void reshape_and_cache(const Tensor& key, const Tensor& value, const Tensor& key
   TORCH_CHECK(chunk == 16 && nh16 * 16 == num_kv_heads * head_size,
               "reshape_and_cache: key_cache must be [num_blocks, num_kv_heads*head_size/16, block_size, 16], got ",
               key_cache.sizes(), " for key ", key.sizes());
-  const bool with_value = value.numel() > 0 && value_cache.numel() > 0;
+  // one of the two without the other would silently leave the V cache stale
+  TORCH_CHECK((value.numel() > 0) == (value_cache.numel() > 0),
+              "reshape_and_cache: value and value_cache must be given together (or both be None)");
+  const bool with_value = value.numel() > 0;
   if (with_value) {
     TORCH_CHECK(value.sizes() == key.sizes(), "reshape_and_cache: value must have the shape of key");
     TORCH_CHECK(value_cache.sizes() == key_cache.sizes(),

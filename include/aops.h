@@ -272,7 +272,9 @@ int aops_moe_combine_f16(const void* y, const int32_t* inverse_idx, const float*
  * multiple of 16 the operator runs on the matrix cores; other page sizes take a generic, slower
  * kernel.  A sequence with context_len <= 0 gets zeros; a context_len beyond
  * max_blocks_per_seq*block_size is cut there.  Block-table entries outside [0, num_blocks) are
- * clamped into it (garbage in, garbage out, no fault).
+ * clamped into it (garbage in, garbage out, no fault).  The workspace size depends on the compute-unit
+ * count of the current device: make the query and the call it sizes with the same device current
+ * (the same holds for the other *_workspace queries of this header).
  * Replaces aclnnPagedAttentionExGetWorkspaceSize + aclnnPagedAttentionEx
  * (reference csrc/ffi/ops.cpp:454-461).
  */

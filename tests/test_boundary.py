@@ -175,6 +175,8 @@ def test_argument_checks_follow_the_reference(ops):
     _raises(ops.reshape_and_cache, key, None, cache, None, slots[:3], match="num_tokens")
     _raises(ops.reshape_and_cache, key, key[0], cache, cache, slots, match="value must be 3D")
     _raises(ops.reshape_and_cache, key, None, torch.zeros(3, 4, 16, 16, dtype=H), None, slots, match="key_cache must be")
+    _raises(ops.reshape_and_cache, key, key, cache, None, slots, match="given together")
+    _raises(ops.reshape_and_cache, key, None, cache, cache, slots, match="given together")
     # paged_attention: shapes the reference assumes silently
     _raises(ops.paged_attention, torch.zeros(2, 8, 128, dtype=H), torch.zeros(4, 16, 128, 8, dtype=H),
             torch.zeros(4, 16, 128, 8, dtype=H), torch.zeros(2, 2, dtype=torch.int32), torch.zeros(2, dtype=torch.int32), match="16")
