@@ -46,6 +46,10 @@ __device__ __forceinline__ int lane_id_fresh() {
 // counted wait stricter, never looser, since vector memory operations complete in order).
 // M0 carries the LDS address of a copy; the compiler reserves that register and warns when it appears in a
 // clobber list, but nothing else in this kernel uses it.
+// Two things therefore hold only as long as the compiler's output keeps them, and tests/test_gmm_waits.py
+// checks both in the assembly of every instantiation at build time (no GPU needed): (1) M0 is written and
+// read by these copy sequences alone, and no register is spilled; (2) between two barriers of the k loop lie
+// exactly the copies the source issues there, and each barrier is directly preceded by its counted wait.
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void dma16(const void* base, uint32_t lane_offset, uint32_t lds_addr) {
