@@ -37,6 +37,7 @@ SOURCES = [
     "grouped_matmul_tiles.hip",
     "grouped_matmul_persistent.hip",
     "matmul_fewrows.hip",
+    "probes.hip",
 ]
 
 # -packed-fp32-ops: keep the compiler from forming packed-fp32 VALU instructions.

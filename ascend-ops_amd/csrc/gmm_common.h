@@ -298,10 +298,13 @@ __device__ __forceinline__ GmmWork gmm_locate(const GmmPlan& p,
 int gmm_launch_tiles(int variant, const f16* x, const f16* w, const int64_t* group_list, f16* y,
                      int64_t rows, int k, int num_experts, int n, hipStream_t stream);
 // Persistent 320x256 kernel; swiglu fuses the activation into the epilogue (y: [rows, n/2]),
-// row_idx != nullptr reads the rows of x through row_idx[j] / idx_div (x has x_rows rows).
+// row_idx != nullptr reads the rows of x through row_idx[j] / idx_div (x has x_rows rows); ldw = elements
+// from one weight row to the next (0 or k: densely packed).
 int gmm_launch_persistent(bool swiglu, const f16* x, const f16* w, const int64_t* group_list, f16* y,
                           int64_t rows, int k, int num_experts, int n, hipStream_t stream,
-                          const int32_t* row_idx, int idx_div, int64_t x_rows);
+                          const int32_t* row_idx, int idx_div, int64_t x_rows, int ldw = 0);
+int gmm_launch_persistent_probe(int parts_off, const f16* x, const f16* w, const int64_t* group_list, f16* y,
+                                int64_t rows, int k, int num_experts, int n, hipStream_t stream);
 
 // Fused gate_up + SwiGLU (row_idx != nullptr: + row gather) on 128 x 128 tiles, or 64 x 64 with
 // `small`; k a multiple of 64.

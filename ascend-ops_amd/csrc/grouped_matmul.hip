@@ -88,6 +88,22 @@ extern "C" int aops_grouped_matmul_variant_f16(int variant, const void* x, const
   return aops_grouped_matmul_impl(x, w, group_list, y, rows, k, num_experts, n, stream, variant);
 }
 
+extern "C" int aops_grouped_matmul_ldw_f16(const void* x, const void* w, int64_t ldw, const int64_t* group_list,
+                                           void* y, int64_t rows, int64_t k, int64_t num_experts, int64_t n,
+                                           void* stream) {
+  using namespace aops;
+  if (rows < 0 || num_experts < 0 || n <= 0 || n % 64 != 0 || k < 256 || k % 128 != 0 || ldw < k || ldw % 8 != 0)
+    return AOPS_ERR_INVALID_ARGUMENT;
+  // per-lane byte offsets inside a weight tile are 32-bit
+  if (rows > 0x7fffffff - 4096 || ldw > (1 << 22) || n > 0x7fffffff || num_experts > (1 << 20))
+    return AOPS_ERR_INVALID_ARGUMENT;
+  if (rows == 0 || num_experts == 0) return AOPS_OK;
+  if (!x || !w || !y || !group_list) return AOPS_ERR_INVALID_ARGUMENT;
+  return gmm_launch_persistent(false, static_cast<const f16*>(x), static_cast<const f16*>(w), group_list,
+                               static_cast<f16*>(y), rows, (int)k, (int)num_experts, (int)n,
+                               static_cast<hipStream_t>(stream), nullptr, 1, 1, (int)ldw);
+}
+
 // Kernel choice of the fused entry points: 0 = persistent 320 x 256 kernel, 1 = 128 x 128 tiles,
 // 2 = 64 x 64 tiles.  Under 96 rows per expert the weights are streamed for little arithmetic and the
 // small tiles win (see the tile choice above); the persistent kernel also needs k % 128 == 0, k >= 256.

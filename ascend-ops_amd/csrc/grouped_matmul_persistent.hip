@@ -65,11 +65,16 @@ __device__ __forceinline__ void dma16(const void* lane_address, uint32_t lds_add
 constexpr int kPlanInts = 2 + kBndCache + 1;  // per-lane record of the group_list scan kept in LDS
 constexpr int kEpiScratchHalfs = 512;         // 1 KiB of LDS per wave for the epilogue's row transposition
 
-template <int MB, int NB, int WN, bool SWIGLU, bool GATHER>
+// PROBE (measurement aid, results wrong by construction): parts of the k loop switched off, so that what
+// the rest costs by itself can be timed: bit 0 = no MFMAs, bit 1 = no activation copies, bit 2 = no weight
+// copies, bit 3 = no LDS fragment reads (the MFMAs then run on registers that never change).  0 = the kernel.
+constexpr int kProbeNoMfma = 1, kProbeNoXCopies = 2, kProbeNoWCopies = 4, kProbeNoFragments = 8;
+
+template <int MB, int NB, int WN, bool SWIGLU, bool GATHER, int PROBE = 0>
 __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kernel(
     const f16* __restrict__ x, const f16* __restrict__ w, const int64_t* __restrict__ group_list,
     f16* __restrict__ y, int64_t rows, int k, int num_experts, int n,
-    const int32_t* __restrict__ row_idx, int idx_div, uint32_t x_rows) {
+    const int32_t* __restrict__ row_idx, int idx_div, uint32_t x_rows, int ldw) {
   constexpr int kWaves = 2 * WN;
   constexpr int BM = 64 * MB;
   constexpr int BN = 32 * NB * WN;
@@ -152,19 +157,22 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   // per-lane offsets of the copies, in bytes (320 rows of at most 2^22 elements: below 2^32)
   const uint32_t off0 = ((uint32_t)lane_row * (uint32_t)k + lane_c * 8) * 2u;
   const uint32_t copy_stride = 8u * kWaves * (uint32_t)k * 2u;
+  // the weight rows are ldw >= k elements apart (rows padded by the caller; ldw == k: densely packed)
+  const uint32_t off0_w = ((uint32_t)lane_row * (uint32_t)ldw + lane_c * 8) * 2u;
+  const uint32_t copy_stride_w = 8u * kWaves * (uint32_t)ldw * 2u;
   uint32_t a_last, b_last;  // offset of this lane's chunk in the last valid row
   uint32_t a_src[GATHER ? kACopies : 1];  // GATHER: offset of this lane's chunk per copy
   // SWIGLU: copy i of the weights fills row blocks 2i (gate rows 32i..32i+31 of the item) and
   // 2i+1 (the up rows d further down): per-lane offset + 32 rows per copy; b_last then holds the
   // number of valid 32-column blocks of the item instead of an offset.
-  const uint32_t off0_glu = (((uint32_t)(lane_row & 31) + (lane_row >= 32 ? (uint32_t)n_out : 0u)) * (uint32_t)k + lane_c * 8) * 2u;
+  const uint32_t off0_glu = (((uint32_t)(lane_row & 31) + (lane_row >= 32 ? (uint32_t)n_out : 0u)) * (uint32_t)ldw + lane_c * 8) * 2u;
   auto set_w_sources = [&](const GmmWork& it) {
     const int lane_s = lane_id_fresh();
     const int lane_row = wave * 8 + ((lane_s >> 3) ^ (wave & 1));
     const int lane_c = (lane_s & 7) ^ (lane_row & 7);
-    b_base = w + ((int64_t)it.expert * n + (int64_t)it.n_tile * BNO) * k;
+    b_base = w + ((int64_t)it.expert * n + (int64_t)it.n_tile * BNO) * ldw;
     const int n_left = min(n_out - it.n_tile * BNO, BNO);
-    b_last = SWIGLU ? (uint32_t)(n_left / 32) : ((uint32_t)(n_left - 1) * (uint32_t)k + lane_c * 8) * 2u;
+    b_last = SWIGLU ? (uint32_t)(n_left / 32) : ((uint32_t)(n_left - 1) * (uint32_t)ldw + lane_c * 8) * 2u;
   };
   auto set_x_sources = [&](const GmmWork& it) {
     const int lane_s = lane_id_fresh();
@@ -188,14 +196,15 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   auto b_offset = [&](int i) -> uint32_t {
     if constexpr (SWIGLU) {
       const uint32_t blk = (uint32_t)i < b_last ? (uint32_t)i : 0u;  // blocks past n: repeat block 0
-      return off0_glu + blk * 64u * (uint32_t)k;
+      return off0_glu + blk * 64u * (uint32_t)ldw;
     } else {
-      return min(off0 + i * copy_stride, b_last);
+      return min(off0_w + i * copy_stride_w, b_last);
     }
   };
   const uint32_t lds_sa = (uint32_t)(uintptr_t)AOPS_LDS_PTR(sa);  // LDS byte addresses of the stages
   const uint32_t lds_sb = (uint32_t)(uintptr_t)AOPS_LDS_PTR(sb);
   auto copy_x = [&](int kt, int stage) {
+    if constexpr (PROBE & kProbeNoXCopies) return;
     const int ko = kt * kBK;
     const uint32_t da = lds_sa + (uint32_t)(stage * BM * kBK + wave * 512) * 2u;
 #pragma unroll
@@ -210,6 +219,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     }
   };
   auto copy_w = [&](int kt, int stage) {
+    if constexpr (PROBE & kProbeNoWCopies) return;
     const int ko = kt * kBK;
     const uint32_t db = lds_sb + (uint32_t)(stage * BN * kBK + wave * 512) * 2u;
 #pragma unroll
@@ -250,11 +260,24 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     constexpr int NF = kSteps * LIVE;  // activation fragments (pairs of MFMAs) of a k tile
     constexpr int kFa = 4;             // activation fragments in flight
     f16x8 fa[LIVE > 0 ? kFa : 1], fb[kSteps][NB];
+    if constexpr (PROBE & kProbeNoFragments) {  // operands the compiler cannot fold: the MFMAs stay
+      const f16x8 one = {1, 1, 1, 1, 1, 1, 1, 1};
+      for (auto& f : fa) {
+        f = one;
+        asm volatile("" : "+v"(f));
+      }
+      for (auto& row : fb)
+        for (auto& f : row) {
+          f = one;
+          asm volatile("" : "+v"(f));
+        }
+    }
     // The XORs are volatile asm: written as expressions they would be hoisted out of the k loop, one
     // address register per (operand, stage, step), and push the accumulators into scratch.
     auto read_fb = [&](auto st_c, auto stage_c) {
       constexpr int ST = decltype(st_c)::value;
       constexpr int STAGE = decltype(stage_c)::value;
+      if constexpr (PROBE & kProbeNoFragments) return;
       uint32_t pb = fb_byte[STAGE];
       if constexpr (ST > 0) asm volatile("v_xor_b32 %0, %1, %2" : "=v"(pb) : "n"(ST << 5), "v"(fb_byte[STAGE]));
 #pragma unroll
@@ -263,7 +286,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     auto read_fa = [&](auto n_c, auto stage_c) {  // fragment n = (row block n / kSteps, k step n % kSteps)
       constexpr int N = decltype(n_c)::value;
       constexpr int STAGE = decltype(stage_c)::value;
-      if constexpr (N >= 0 && N < NF) {
+      if constexpr (N >= 0 && N < NF && !(PROBE & kProbeNoFragments)) {
         constexpr int ST = N % kSteps;
         uint32_t pa = fa_byte[STAGE];
         if constexpr (ST > 0) asm volatile("v_xor_b32 %0, %1, %2" : "=v"(pa) : "n"(ST << 5), "v"(fa_byte[STAGE]));
@@ -272,7 +295,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     };
     auto mma = [&](auto n_c) {
       constexpr int N = decltype(n_c)::value;
-      if constexpr (N >= 0 && N < NF) {
+      if constexpr (N >= 0 && N < NF && !(PROBE & kProbeNoMfma)) {
 #pragma unroll
         for (int j = 0; j < NB; ++j)
           acc[N / kSteps][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[N % kSteps][j], fa[N % kFa],
@@ -462,10 +485,11 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
 }
 
-template <int MB, int NB, int WN, bool SWIGLU, bool GATHER = false>
+template <int MB, int NB, int WN, bool SWIGLU, bool GATHER = false, int PROBE = 0>
 static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* group_list, f16* y,
                                  int64_t rows, int k, int num_experts, int n, hipStream_t stream,
-                                 const int32_t* row_idx = nullptr, int idx_div = 1, int64_t x_rows = 1) {
+                                 const int32_t* row_idx = nullptr, int idx_div = 1, int64_t x_rows = 1, int ldw = 0) {
+  if (ldw == 0) ldw = k;  // densely packed weight rows
   constexpr int BM = 64 * MB;
   constexpr int BN = 32 * NB * WN;
   constexpr int kWaves = 2 * WN;
@@ -481,12 +505,12 @@ static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* grou
   int64_t grid = cus < max_work ? cus : max_work;
   grid = grid / kXcds * kXcds;
   if (grid < kXcds) grid = kXcds;
-  auto kernel = grouped_matmul_persistent_kernel<MB, NB, WN, SWIGLU, GATHER>;
+  auto kernel = grouped_matmul_persistent_kernel<MB, NB, WN, SWIGLU, GATHER, PROBE>;
   static std::atomic<uint64_t> lds_allowed{0};  // per device
   if (const hipError_t le = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLds, lds_allowed); le != hipSuccess)
     return record_launch_status(le);
   kernel<<<(unsigned)grid, 2 * WN * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts,
-                                                          n, row_idx, idx_div, (uint32_t)x_rows);
+                                                          n, row_idx, idx_div, (uint32_t)x_rows, ldw);
   return record_launch_status(hipGetLastError());
 }
 
@@ -512,22 +536,42 @@ static bool gmm_prefer_256_rows(int64_t rows, int64_t num_experts, int64_t n_out
 
 int gmm_launch_persistent(bool swiglu, const f16* x, const f16* w, const int64_t* group_list, f16* y,
                           int64_t rows, int k, int num_experts, int n, hipStream_t stream,
-                          const int32_t* row_idx, int idx_div, int64_t x_rows) {
+                          const int32_t* row_idx, int idx_div, int64_t x_rows, int ldw) {
   const int64_t n_out_tiles = swiglu ? (n / 2 + 127) / 128 : (n + 255) / 256;
   const bool small = gmm_prefer_256_rows(rows, num_experts, n_out_tiles, device_cu_count());
   if (row_idx) {  // only the fused gate_up form gathers
     if (small)
       return gmm_persistent_launch<4, 2, 4, true, true>(x, w, group_list, y, rows, k, num_experts, n, stream,
-                                                        row_idx, idx_div, x_rows);
+                                                        row_idx, idx_div, x_rows, ldw);
     return gmm_persistent_launch<5, 2, 4, true, true>(x, w, group_list, y, rows, k, num_experts, n, stream,
-                                                      row_idx, idx_div, x_rows);
+                                                      row_idx, idx_div, x_rows, ldw);
   }
   if (swiglu) {
-    if (small) return gmm_persistent_launch<4, 2, 4, true>(x, w, group_list, y, rows, k, num_experts, n, stream);
-    return gmm_persistent_launch<5, 2, 4, true>(x, w, group_list, y, rows, k, num_experts, n, stream);
+    if (small)
+      return gmm_persistent_launch<4, 2, 4, true>(x, w, group_list, y, rows, k, num_experts, n, stream, nullptr, 1, 1, ldw);
+    return gmm_persistent_launch<5, 2, 4, true>(x, w, group_list, y, rows, k, num_experts, n, stream, nullptr, 1, 1, ldw);
   }
-  if (small) return gmm_persistent_launch<4, 2, 4, false>(x, w, group_list, y, rows, k, num_experts, n, stream);
-  return gmm_persistent_launch<5, 2, 4, false>(x, w, group_list, y, rows, k, num_experts, n, stream);
+  if (small)
+    return gmm_persistent_launch<4, 2, 4, false>(x, w, group_list, y, rows, k, num_experts, n, stream, nullptr, 1, 1, ldw);
+  return gmm_persistent_launch<5, 2, 4, false>(x, w, group_list, y, rows, k, num_experts, n, stream, nullptr, 1, 1, ldw);
+}
+
+// The 320 x 256 kernel with parts of its k loop switched off (see PROBE): a measurement aid.
+int gmm_launch_persistent_probe(int parts_off, const f16* x, const f16* w, const int64_t* group_list, f16* y,
+                                int64_t rows, int k, int num_experts, int n, hipStream_t stream) {
+  switch (parts_off) {
+#define AOPS_PROBE_CASE(P) \
+  case (P):                \
+    return gmm_persistent_launch<5, 2, 4, false, false, (P)>(x, w, group_list, y, rows, k, num_experts, n, stream);
+    AOPS_PROBE_CASE(kProbeNoMfma | kProbeNoFragments)                       // 9: copies and barriers only
+    AOPS_PROBE_CASE(kProbeNoMfma | kProbeNoFragments | kProbeNoXCopies)     // 11: weight copies only
+    AOPS_PROBE_CASE(kProbeNoMfma | kProbeNoFragments | kProbeNoWCopies)     // 13: activation copies only
+    AOPS_PROBE_CASE(kProbeNoXCopies | kProbeNoWCopies)                      // 6: MFMAs and fragment reads only
+    AOPS_PROBE_CASE(kProbeNoXCopies | kProbeNoWCopies | kProbeNoFragments)  // 14: MFMAs only
+#undef AOPS_PROBE_CASE
+    default:
+      return AOPS_ERR_INVALID_ARGUMENT;
+  }
 }
 
 }  // namespace aops

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ascend910a_extras operator set on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|norm|cache|rope|mlp|moe|moe_gate_up|moe_down|pa_more|dense|scaled,...] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|norm|cache|rope|mlp|moe|moe_gate_up|moe_down|pa_more|dense|gmm_probe|scaled,...] [--no-cpu]
 
 A "step" is one paged_attention decode call over the batch of BASELINE.json configs[4]
 (64 sequences, 32 query / 8 kv heads, head_dim 128, contexts ~U[512, 4096], block 128): the
@@ -814,6 +814,90 @@ def bench_dense(L, R, dev):
     return e
 
 
+def bench_gmm_probe(L, R, dev):
+    """Where the time of the MoE GEMMs goes, from kernels in the library alone: the persistent grouped-matmul kernel
+    on configs[3] with parts of its k loop switched off (aops_grouped_matmul_probe_f16), and a pure read stream
+    with the access pattern of its weight copies next to a linear stream of the same bytes
+    (aops_probe_read_stream).  Results of the switched-off forms are wrong by construction; only times count."""
+    import torch
+
+    E, hidden, inter, tokens, topk = 128, 2048, 768, 4096, 8
+    rows = tokens * topk
+    torch.manual_seed(0)
+    gl = R.make_group_list(torch.randint(0, E, (rows,)), E).to(dev)
+    out = []
+    for which, K, N in (("gate_up", hidden, 2 * inter), ("down", inter, hidden)):
+        g = torch.Generator(device=dev).manual_seed(1)
+        sets = 2
+        xs = [torch.randn(rows, K, generator=g, device=dev, dtype=torch.float16) for _ in range(sets)]
+        ws = [torch.randn(E, N, K, generator=g, device=dev, dtype=torch.float16) * 0.02 for _ in range(sets)]
+        ys = [torch.empty(rows, N, device=dev, dtype=torch.float16) for _ in range(sets)]
+        flops = 2 * rows * K * N
+        alg = rows * K * 2 + E * N * K * 2 + rows * N * 2 + E * 8
+
+        def timed(parts_off):
+            if parts_off == 0:
+                calls = [(lambda i=i: L.check(L.lib.aops_grouped_matmul_variant_f16(
+                    6, xs[i].data_ptr(), ws[i].data_ptr(), gl.data_ptr(), ys[i].data_ptr(), rows, K, E, N, L.stream())))
+                    for i in range(sets)]
+            else:
+                calls = [(lambda i=i: L.check(L.lib.aops_grouped_matmul_probe_f16(
+                    parts_off, xs[i].data_ptr(), ws[i].data_ptr(), gl.data_ptr(), ys[i].data_ptr(), rows, K, E, N,
+                    L.stream()))) for i in range(sets)]
+            return time_graph(calls, min_launches=40, trials=3)
+
+        for parts_off, what in ((0, "whole kernel"), (9, "operand copies and barriers only"), (11, "weight copies only"),
+                                (13, "activation copies only"), (6, "MFMAs and LDS fragment reads only"), (14, "MFMAs only")):
+            med, mn = timed(parts_off)
+            e = entry("grouped_matmul_probe", f"probe 4: MoE {which}, {what}", f"x [{rows},{K}] @ w [{E},{K},{N}] f16",
+                      "mfma", alg, flops, med, mn, None, None, 1,
+                      None if parts_off == 0 else "parts of the k loop switched off: results wrong by construction, time only")
+            e["parts_off"] = parts_off
+            out.append(e)
+        # the same GEMM on weights whose rows are padded by one cache line (aops_grouped_matmul_ldw_f16): what the
+        # power-of-two row stride of the reference's layout costs
+        ldw = K + 64
+        wps = []
+        for i in range(sets):
+            wp = torch.zeros(E, N, ldw, device=dev, dtype=torch.float16)
+            wp[:, :, :K] = ws[i]
+            wps.append(wp)
+        y_pad = torch.empty(rows, N, device=dev, dtype=torch.float16)
+        L.check(L.lib.aops_grouped_matmul_ldw_f16(xs[0].data_ptr(), wps[0].data_ptr(), ldw, gl.data_ptr(), y_pad.data_ptr(),
+                                                  rows, K, E, N, L.stream()))
+        L.check(L.lib.aops_grouped_matmul_variant_f16(6, xs[0].data_ptr(), ws[0].data_ptr(), gl.data_ptr(), ys[0].data_ptr(),
+                                                      rows, K, E, N, L.stream()))
+        assert torch.equal(y_pad, ys[0]), "padded weight rows must give the same bits"
+        calls = [(lambda i=i: L.check(L.lib.aops_grouped_matmul_ldw_f16(
+            xs[i].data_ptr(), wps[i].data_ptr(), ldw, gl.data_ptr(), ys[i].data_ptr(), rows, K, E, N, L.stream())))
+            for i in range(sets)]
+        med, mn = time_graph(calls, min_launches=40, trials=3)
+        out.append(entry("grouped_matmul_ldw", f"probe 4: MoE {which}, weight rows padded to {2 * ldw} bytes (extension)",
+                         f"x [{rows},{K}] @ w [{E},{K},{N}] f16, row stride {ldw}", "mfma", alg, flops, med, mn, None, None, 1,
+                         "same kernel and same bits as the whole-kernel line; the caller pads the static weights once"))
+        del wps, y_pad
+        # the weight bytes of this GEMM as a pure read stream: the kernel's pattern, longer pieces, and linear
+        wbytes = E * N * K * 2
+        sink = torch.zeros(1, dtype=torch.float32, device=dev)
+        for seg, row_bytes, what in ((128, 2 * K, f"128-byte pieces one weight row ({2 * K} B) apart, as the kernel copies them"),
+                                     (256, 2 * K, "256-byte pieces one weight row apart"),
+                                     (512, 2 * K, "512-byte pieces one weight row apart"),
+                                     (128, 2 * K + 128, f"128-byte pieces {2 * K + 128} B apart (what a row padded by one line would give)"),
+                                     (1024, 1024, "the same bytes read linearly (1 KiB per row of the probe)")):
+            if row_bytes % seg != 0:
+                continue
+            nrows = wbytes // row_bytes // 128 * 128
+            calls = [(lambda i=i: L.check(L.lib.aops_probe_read_stream(ws[i].data_ptr(), nrows, row_bytes, seg,
+                                                                        sink.data_ptr(), L.stream()))) for i in range(sets)]
+            med, mn = time_graph(calls, min_launches=40, trials=3)
+            out.append(entry("read_stream_probe", f"probe 4: weights of MoE {which} as a read stream, {what}",
+                             f"[{nrows},{row_bytes}] bytes, 128 rows per workgroup", "hbm", nrows * row_bytes, 0, med, mn,
+                             None, None, 1))
+        del xs, ws, ys
+        torch.cuda.empty_cache()
+    return out
+
+
 def kernel_source_digest():
     """Digest of the paged-attention kernels' source: the recorded HBM-traffic figure names the digest it was
     measured on and is dropped when the source has changed since."""
@@ -902,6 +986,7 @@ def main():
         for tag, fn in (("moe_gate_up", lambda: bench_moe_one(L, ops, R, dev, "gate_up")),
                         ("moe_down", lambda: bench_moe_one(L, ops, R, dev, "down")),
                         ("dense", lambda: bench_dense(L, R, dev)),
+                        ("gmm_probe", lambda: bench_gmm_probe(L, R, dev)),
                         ("pa_more", lambda: bench_pa_more(L, R, dev, cpu))):
             if tag in want:
                 run(tag, fn)
@@ -939,6 +1024,7 @@ def main():
         run("moe_down", lambda: bench_moe_one(L, ops, R, dev, "down"))
     run("pa_more", lambda: bench_pa_more(L, R, dev, cpu))
     run("dense", lambda: bench_dense(L, R, dev))
+    run("gmm_probe", lambda: bench_gmm_probe(L, R, dev))
     run("scaled", lambda: [
         bench_add_rms_norm(L, ops, R, dev, False, 16384, "1 scaled x128: add_rms_norm",
                            "scaled shape: shows the kernel's asymptotic bandwidth, not a BASELINE config"),

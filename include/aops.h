@@ -171,6 +171,23 @@ int aops_grouped_matmul_variant_f16(int variant, const void* x, const void* w,
                                     int64_t num_experts, int64_t n, void* stream);
 
 /*
+ * aops_grouped_matmul_f16 for weights whose rows are padded: row r of expert e starts at element
+ * (e * n + r) * ldw of w, ldw >= k a multiple of 8, and only its first k elements are read (in torch terms the
+ * logical [E, K, N] tensor with stride(1) == 1, stride(2) == ldw, stride(0) == n * ldw).  Why a caller might pad:
+ * with k * 2 bytes a power of two (k = 2048: 4 KiB) the 128-byte pieces that a weight tile takes from 256
+ * consecutive rows fall into the same few memory channels; a pure read stream of that pattern runs at 4.8 TB/s
+ * and at 7.0 TB/s with rows 4224 bytes apart (ldw = k + 64; aops_probe_read_stream shows both).  The grouped
+ * matmul itself gains little from it (configs of 32768 routed rows, 128 experts, k = 2048: 2 %), because its
+ * operand copies are bound by the number of cache lines in flight per CU, not by the weight stream alone; the
+ * entry point exists so that this can be measured.  Runs the persistent 320 x 256 kernel for every problem
+ * size: k must be a multiple of 128 from 256 on, n a multiple of 64.  Same bits as aops_grouped_matmul_f16
+ * with that kernel on the unpadded weights.
+ * No counterpart in the reference, whose binding insists on stride(2) == K (reference csrc/ffi/ops.cpp:171-172).
+ */
+int aops_grouped_matmul_ldw_f16(const void* x, const void* w, int64_t ldw, const int64_t* group_list, void* y,
+                                int64_t rows, int64_t k, int64_t num_experts, int64_t n, void* stream);
+
+/*
  * Dense NT matmul: y = f16( x (fp32 accumulate) @ w^T ), x: [m, k], w: [n, k], y: [m, n]; the
  * grouped matmul with one group that holds every row (no group_list needed).  k and n must be
  * multiples of 64.
@@ -320,6 +337,30 @@ int aops_paged_attention_noalloc_f16(const void* q, const void* key_cache, const
  * No counterpart in the reference.
  */
 int aops_empty_launch(int64_t workgroups, int threads, void* stream);
+
+/*
+ * Measurement aid: a pure read stream with the access pattern of a GEMM operand copy.  buf is a
+ * [rows, row_bytes] byte matrix (rows a multiple of 128); every workgroup owns 128 consecutive rows and
+ * walks along them in steps of seg_bytes (128, 256, 512 or 1024, dividing row_bytes) per row.  With
+ * seg_bytes = 128 and row_bytes = 2 * k this is how the weight tiles of the grouped matmul are fetched;
+ * with row_bytes == seg_bytes every workgroup reads one contiguous block (a linear stream).  sink: 4 bytes
+ * of device memory that are never written for finite data.  Bandwidth = rows * row_bytes / duration.
+ * No counterpart in the reference.
+ */
+int aops_probe_read_stream(const void* buf, int64_t rows, int64_t row_bytes, int64_t seg_bytes, void* sink,
+                           void* stream);
+
+/*
+ * Measurement aid: the persistent 320 x 256 kernel of aops_grouped_matmul_f16 (k % 128 == 0, k >= 256)
+ * with parts of its k loop switched off, to time what the rest costs by itself.  parts_off: 9 = operand
+ * copies and barriers only (no MFMAs, no LDS fragment reads), 11 = weight copies only, 13 = activation
+ * copies only, 6 = MFMAs and fragment reads only (no copies), 14 = MFMAs only; anything else returns
+ * AOPS_ERR_INVALID_ARGUMENT.  y is written with values that are wrong by construction.
+ * No counterpart in the reference.
+ */
+int aops_grouped_matmul_probe_f16(int parts_off, const void* x, const void* w, const int64_t* group_list,
+                                  void* y, int64_t rows, int64_t k, int64_t num_experts, int64_t n,
+                                  void* stream);
 
 /*
  * Device summary (CU count, LDS, L2, memory size, clocks) written as text into buf

@@ -6,7 +6,7 @@ the compiler's own wait-count pass does not see the copies; the kernel waits for
 ``s_waitcnt`` immediates in front of bare ``s_barrier`` instructions:
 
 * barrier B of a k tile follows the tile's activation copies (``kACopies`` per wave) and is preceded by a wait
-  on LDS reads only;
+  on LDS reads only ("preceded": in the same basic block, with nothing that touches memory or LDS in between);
 * barrier A follows the weight copies (``kBCopies`` per wave) issued after barrier B and is preceded by
   ``s_waitcnt vmcnt(kBCopies) lgkmcnt(0)``: everything but the weight copies just issued has landed.  Vector
   memory operations complete in order, so other memory operations in between can only make that wait stricter;
@@ -26,7 +26,9 @@ import collections
 import re
 
 COPY = "global_load_lds_dwordx4"
-_KERNEL = re.compile(r"^_ZN4aops32grouped_matmul_persistent_kernelILi(\d+)ELi(\d+)ELi(\d+)ELb([01])ELb([01])E")
+_MEMORY = ("global_", "ds_", "buffer_", "scratch_", "flat_", "s_load", "s_buffer_load", "s_store", "s_scratch")
+# <MB, NB, WN, SWIGLU, GATHER, PROBE>; the measurement builds (PROBE != 0) leave copies out on purpose and are not checked
+_KERNEL = re.compile(r"^_ZN4aops32grouped_matmul_persistent_kernelILi(\d+)ELi(\d+)ELi(\d+)ELb([01])ELb([01])ELi0EE")
 
 
 def kernels(asm_text: str):
@@ -78,6 +80,7 @@ def scan_kernel(name: str, body) -> tuple:
             labels[m.group(1)] = len(ins)
         elif code.startswith("\t") and not code.strip().startswith("."):
             ins.append(code.strip().replace(",", " ").split())
+    label_at = set(labels.values())
     preds = collections.defaultdict(list)
     for i, t in enumerate(ins):
         if t[0] not in ("s_branch", "s_endpgm", "s_setpc_b64") and i + 1 < len(ins):
@@ -108,10 +111,16 @@ def scan_kernel(name: str, body) -> tuple:
         if t[0] != "s_barrier":
             continue
         barriers += 1
-        if i == 0 or ins[i - 1][0] != "s_waitcnt":
-            findings.append(f"{name}: s_barrier at instruction {i} without an s_waitcnt directly in front")
+        # the wait belongs to the barrier: same basic block, and nothing that touches memory or LDS in between
+        # (register moves the compiler places there are harmless)
+        w = i - 1
+        while w >= 0 and ins[w][0] != "s_waitcnt" and not ins[w][0].startswith(_MEMORY) and \
+                not ins[w][0].startswith(("s_cbranch", "s_branch", "s_barrier")) and (w + 1) not in label_at and i - w < 24:
+            w -= 1
+        if w < 0 or ins[w][0] != "s_waitcnt" or any(j in label_at for j in range(w + 1, i + 1)):
+            findings.append(f"{name}: s_barrier at instruction {i} without an s_waitcnt in front")
             continue
-        wait = _wait_fields(ins[i - 1])
+        wait = _wait_fields(ins[w])
         counts, at_entry = set(), set()
         seen, stack = set(), [(p, 0) for p in preds[i]]
         while stack:

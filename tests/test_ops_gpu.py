@@ -336,6 +336,72 @@ def test_grouped_matmul_every_kernel(ops, dev, variant, rows, K, N, E, counts):
     assert torch.all(y[end:] == 5.0)
 
 
+@pytest.mark.parametrize("rows,K,N,E,pad,counts", [
+    (1500, 256, 192, 6, 64, None),
+    (900, 2048, 320, 3, 64, [0, 650, 250]),       # the row length whose power-of-two stride the padding is for
+    (640, 384, 64, 2, 8, [320, 300]),             # the smallest padding; rows past the last group
+])
+def test_grouped_matmul_with_padded_weight_rows(dev, rows, K, N, E, pad, counts):
+    """aops_grouped_matmul_ldw_f16: weight rows ldw = K + pad elements apart.  The padding holds NaN and must never be
+    read into a product; the result equals the persistent kernel's on the unpadded weights bit for bit (same kernel,
+    same order of operations) and the oracle within tolerance; rows past the last group stay untouched."""
+    lib = cabi.lib()
+    x, w, gl = _gmm_case(rows, K, N, E, seed=31, counts=counts)
+    end = int(gl[-1])
+    storage = w.transpose(1, 2).contiguous()                       # [E, N, K]
+    padded = torch.full((E, N, K + pad), float("nan"), dtype=H)
+    padded[:, :, :K] = storage
+    xd, wd, pd, gd = x.to(dev), storage.to(dev), padded.to(dev), gl.to(dev)
+    y = torch.full((rows, N), 5.0, dtype=H, device=dev)
+    y_ref = torch.full((rows, N), 5.0, dtype=H, device=dev)
+    assert lib.aops_grouped_matmul_ldw_f16(xd.data_ptr(), pd.data_ptr(), K + pad, gd.data_ptr(), y.data_ptr(), rows, K, E,
+                                           N, cabi.stream(dev)) == 0
+    assert lib.aops_grouped_matmul_variant_f16(6, xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y_ref.data_ptr(), rows, K,
+                                               E, N, cabi.stream(dev)) == 0
+    assert torch.equal(y, y_ref)
+    torch.testing.assert_close(y.cpu()[:end].float(), R.grouped_matmul_ref(x, w, gl)[:end].float(), **GMM_TOL)
+    assert torch.all(y[end:] == 5.0)
+    # ldw == K is the unpadded operator; a stride below K, or one that breaks the 16-byte alignment of the rows, is refused
+    y2 = torch.full((rows, N), 5.0, dtype=H, device=dev)
+    assert lib.aops_grouped_matmul_ldw_f16(xd.data_ptr(), wd.data_ptr(), K, gd.data_ptr(), y2.data_ptr(), rows, K, E, N,
+                                           cabi.stream(dev)) == 0
+    assert torch.equal(y2, y_ref)
+    for bad in (K - 8, K + 4):
+        assert lib.aops_grouped_matmul_ldw_f16(xd.data_ptr(), pd.data_ptr(), bad, gd.data_ptr(), y.data_ptr(), rows, K, E,
+                                               N, cabi.stream(dev)) == -1
+
+
+def test_measurement_aids_run_and_leave_their_surroundings_alone(dev):
+    """The probe entry points (parts of the persistent kernel's k loop switched off; a pure read stream) are
+    measurement aids whose results mean nothing, but they must run to completion, refuse what they do not serve, write
+    nothing outside y and read nothing outside their operands (guard regions keep their contents)."""
+    lib = cabi.lib()
+    rows, K, N, E = 700, 256, 192, 5
+    x, w, gl = _gmm_case(rows, K, N, E, seed=2, counts=[300, 0, 1, 330, 69])
+    xd, wd, gd = x.to(dev), w.transpose(1, 2).contiguous().to(dev), gl.to(dev)
+    y = torch.full((rows + 2, N), 7.0, dtype=H, device=dev)        # one guard row on either side
+    for parts_off in (9, 11, 13, 6, 14):
+        assert lib.aops_grouped_matmul_probe_f16(parts_off, xd.data_ptr(), wd.data_ptr(), gd.data_ptr(),
+                                                 y[1:].data_ptr(), rows, K, E, N, cabi.stream(dev)) == 0
+    torch.cuda.synchronize()
+    assert torch.all(y[0] == 7.0) and torch.all(y[-1] == 7.0)
+    for bad in (0, 1, 7, 15, -1):
+        assert lib.aops_grouped_matmul_probe_f16(bad, xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y[1:].data_ptr(),
+                                                 rows, K, E, N, cabi.stream(dev)) == -1
+    assert lib.aops_grouped_matmul_probe_f16(9, xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y[1:].data_ptr(),
+                                             rows, 192, E, N, cabi.stream(dev)) == -1    # k the kernel does not take
+    buf = torch.ones(256 * 1024, dtype=torch.uint8, device=dev)
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    for seg, row_bytes in ((128, 1024), (256, 512), (512, 512), (1024, 1024), (128, 128)):
+        assert lib.aops_probe_read_stream(buf.data_ptr(), buf.numel() // row_bytes, row_bytes, seg, sink.data_ptr(),
+                                          cabi.stream(dev)) == 0
+    torch.cuda.synchronize()
+    assert float(sink[0]) == 0.0
+    assert lib.aops_probe_read_stream(buf.data_ptr(), 100, 1024, 128, sink.data_ptr(), cabi.stream(dev)) == -1   # rows % 128
+    assert lib.aops_probe_read_stream(buf.data_ptr(), 256, 1024, 96, sink.data_ptr(), cabi.stream(dev)) == -1    # piece size
+    assert lib.aops_probe_read_stream(buf.data_ptr(), 256, 640, 256, sink.data_ptr(), cabi.stream(dev)) == -1    # not dividing
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_grouped_matmul_persistent_kernel_random_shapes(ops, dev, seed):
     """The persistent kernel (variant 6) on seeded random problems: group sizes from empty to several tiles (every
