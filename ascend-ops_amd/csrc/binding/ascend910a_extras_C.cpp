@@ -226,10 +226,13 @@ void reshape_and_cache(const Tensor& key, const Tensor& value, const Tensor& key
   TORCH_CHECK(chunk == 16 && nh16 * 16 == num_kv_heads * head_size,
               "reshape_and_cache: key_cache must be [num_blocks, num_kv_heads*head_size/16, block_size, 16], got ",
               key_cache.sizes(), " for key ", key.sizes());
-  // one of the two without the other would silently leave the V cache stale
-  TORCH_CHECK((value.numel() > 0) == (value_cache.numel() > 0),
+  // "None" arrives as an empty 1-D tensor; a batch of zero tokens is an empty 3-D value and still "given".
+  // One of the two without the other would silently leave the V cache stale.
+  const bool value_given = value.numel() > 0 || value.dim() == 3;
+  const bool value_cache_given = value_cache.numel() > 0 || value_cache.dim() == 4;
+  TORCH_CHECK(value_given == value_cache_given,
               "reshape_and_cache: value and value_cache must be given together (or both be None)");
-  const bool with_value = value.numel() > 0;
+  const bool with_value = value_given;
   if (with_value) {
     TORCH_CHECK(value.sizes() == key.sizes(), "reshape_and_cache: value must have the shape of key");
     TORCH_CHECK(value_cache.sizes() == key_cache.sizes(),

@@ -633,58 +633,51 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_balanced(
   const int head0 = g * ge.group + v * ge.wg_heads;
   const int nh = min(ge.wg_heads, ge.group - v * ge.wg_heads);
   const int max_len = ge.max_blocks_per_seq * ge.block_size;
-  if (bs > kWave) {
+  const bool planned = bs > kWave;  // the partition lives in LDS (pa_block_plan), else in the lanes (pa_units)
+  const int* lds_plan = nullptr;
+  PaUnits pu = {0, 0, 0, 0};
+  int total, next_b = 0;
+  if (planned) {
     extern __shared__ __attribute__((aligned(16))) unsigned char pa_lds[];
-    int* lds_plan = reinterpret_cast<int*>(pa_lds + pa_q_lds_halfs<D, NSUB>() * sizeof(f16)) +
-                    kPaWaves * ge.merge_heads * (D + 2);
-    pa_block_plan(context_lens, bs, max_len, (int)gridDim.x, w, lds_plan, plan, w == 0 && blockIdx.y == 0);
-    const int total = lds_plan[2 * bs];
-    const int wgs = min((int)gridDim.x, total);
-    if (w >= wgs) return;
-    const int lo = (int)((int64_t)w * total / wgs);
-    const int hi = (int)((int64_t)(w + 1) * total / wgs);
-    int cur = lo;
-    int b = lds_plan[2 * bs + 1];
-    while (cur < hi && b < bs) {
-      const int before = lds_plan[b];
-      const int len = lds_plan[bs + b];
-      const int units = (len + kPaUnit - 1) / kPaUnit;
-      if (units > 0) {
-        const int seg_end = min(hi, before + units);
-        const int tok0 = (cur - before) * kPaUnit;
-        const int tok1 = min((seg_end - before) * kPaUnit, len);
-        const int first = pa_share_of(before, wgs, total);
-        const bool whole = pa_share_of(before + units - 1, wgs, total) == first;
-        pa_process_chunk<D, NSUB>(q, key_cache, value_cache, block_tables, part_o, part_ml, out, whole, b, g,
-                                  head0, nh, len, tok0, tok1 - tok0, w - first, ge);
-        cur = seg_end;
-        if (cur < hi) __syncthreads();  // the LDS arrays of the chunk are reused
-      }
-      ++b;
-    }
-    return;
+    int* plan_w = reinterpret_cast<int*>(pa_lds + pa_q_lds_halfs<D, NSUB>() * sizeof(f16)) +
+                  kPaWaves * ge.merge_heads * (D + 2);
+    pa_block_plan(context_lens, bs, max_len, (int)gridDim.x, w, plan_w, plan, w == 0 && blockIdx.y == 0);
+    lds_plan = plan_w;
+    total = lds_plan[2 * bs];
+    next_b = lds_plan[2 * bs + 1];  // the sequence that holds the share's first unit
+  } else {
+    pu = pa_units(context_lens, bs, max_len);
+    total = pu.total;
   }
-  const PaUnits pu = pa_units(context_lens, bs, max_len);
   // no more shares than units: every share then holds at least one unit, and the shares of a
   // sequence are consecutive
-  const int wgs = min((int)gridDim.x, pu.total);
+  const int wgs = min((int)gridDim.x, total);
   if (w >= wgs) return;
-  const int lo = (int)((int64_t)w * pu.total / wgs);
-  const int hi = (int)((int64_t)(w + 1) * pu.total / wgs);
+  const int lo = (int)((int64_t)w * total / wgs);
+  const int hi = (int)((int64_t)(w + 1) * total / wgs);
   int cur = lo;
   while (cur < hi) {
-    // the sequence that holds unit cur (exactly one lane)
-    const uint64_t hit = __ballot(pu.units > 0 && pu.before <= cur && cur < pu.before + pu.units);
-    if (hit == 0) break;  // cannot happen: the units of the sequences tile [0, total)
-    const int b = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(hit));
-    const int before = __builtin_amdgcn_readlane(pu.before, b);
-    const int units = __builtin_amdgcn_readlane(pu.units, b);
-    const int len = __builtin_amdgcn_readlane(pu.len, b);
+    // the sequence that holds unit cur
+    int b, before, len;
+    if (planned) {
+      while (next_b < bs && lds_plan[bs + next_b] <= 0) ++next_b;  // empty sequences hold no unit
+      if (next_b >= bs) break;  // cannot happen: the units of the sequences tile [0, total)
+      b = next_b++;
+      before = lds_plan[b];
+      len = lds_plan[bs + b];
+    } else {
+      const uint64_t hit = __ballot(pu.units > 0 && pu.before <= cur && cur < pu.before + pu.units);  // one lane
+      if (hit == 0) break;  // cannot happen either
+      b = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(hit));
+      before = __builtin_amdgcn_readlane(pu.before, b);
+      len = __builtin_amdgcn_readlane(pu.len, b);
+    }
+    const int units = (len + kPaUnit - 1) / kPaUnit;
     const int seg_end = min(hi, before + units);
     const int tok0 = (cur - before) * kPaUnit;
     const int tok1 = min((seg_end - before) * kPaUnit, len);
-    const int first = pa_share_of(before, wgs, pu.total);
-    const bool whole = pa_share_of(before + units - 1, wgs, pu.total) == first;
+    const int first = pa_share_of(before, wgs, total);
+    const bool whole = pa_share_of(before + units - 1, wgs, total) == first;
     pa_process_chunk<D, NSUB>(q, key_cache, value_cache, block_tables, part_o, part_ml, out, whole, b, g,
                               head0, nh, len, tok0, tok1 - tok0, w - first, ge);
     cur = seg_end;

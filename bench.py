@@ -487,7 +487,7 @@ def _moe_glue_entries(L, dev, E, hidden, tokens, topk):
                                                         gl.data_ptr(), ws.data_ptr(), ws_bytes, L.stream()))
     med, mn = time_graph([sort_call], min_launches=100)
     out.append(entry("moe_sort", "4: routing sort (extension)", f"ids [{tokens},{topk}] int32, {E} experts", "hbm",
-                     n * 4 * 3 + E * 8, 0, med, mn, None, None, 1, "three launches: histogram, scan, stable scatter"))
+                     n * 4 * 3 + E * 8, 0, med, mn, None, None, 1, "two launches: per-slice histograms, then a scatter whose waves scan the histograms themselves (stable)"))
     n_sets = n_sets_for(n * hidden * 2 * 2)
     xs = [torch.empty(n, hidden, dtype=torch.float16, device=dev) for _ in range(n_sets)]
     med, mn = time_graph([(lambda i=i: L.check(L.lib.aops_moe_gather_f16(x.data_ptr(), s_idx.data_ptr(), gl.data_ptr(),

@@ -23,7 +23,11 @@ H = torch.float16
         (63, 1, 2, False),
         (77, 6, 300, True),        # more experts than lanes of a wave
         (513, 1, 4095, False),     # largest expert count
-        (20000, 4, 3, False),      # long runs of equal ids
+        (20000, 4, 3, False),      # long runs of equal ids; more than 65536 ids: histogram, scan and scatter kernels
+        (8192, 8, 255, True),      # 65536 ids, 256 buckets: the largest table of the two-launch sort
+        (8193, 8, 255, True),      # one token more: the three-kernel sort
+        (3000, 3, 256, True),      # 257 buckets: the three-kernel sort
+        (1111, 7, 64, True),       # last workgroup with idle waves and a ragged last slice
     ],
 )
 def test_moe_sort_matches_a_stable_sort_exactly(dev, tokens, topk, E, invalid):
