@@ -145,17 +145,19 @@ __global__ __launch_bounds__(kMoeWaves* kWave) void moe_scatter_kernel(
     int before[kPer], total[kPer];
 #pragma unroll
     for (int j = 0; j < kPer; ++j) before[j] = total[j] = 0;
-    for (int s0 = 0; s0 < num_slices; s0 += 8) {  // eight rows of loads in flight
-      int c[8][kPer];
+    // 32 rows of loads in flight: the histograms of a prefill batch (64 slices) arrive in two round trips
+    constexpr int kRows = 32;
+    for (int s0 = 0; s0 < num_slices; s0 += kRows) {
+      int c[kRows][kPer];
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
+      for (int u = 0; u < kRows; ++u)
 #pragma unroll
         for (int j = 0; j < kPer; ++j) {
           const int e = lane + kWave * j;
           c[u][j] = (s0 + u < num_slices && e < buckets) ? counts[(int64_t)(s0 + u) * buckets + e] : 0;
         }
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
+      for (int u = 0; u < kRows; ++u)
 #pragma unroll
         for (int j = 0; j < kPer; ++j) {
           total[j] += c[u][j];

@@ -233,9 +233,12 @@ __device__ __forceinline__ void pa_accumulate(const PaRegs<PaDims<D>::kSlices>& 
   }
 }
 
-// LDS of the main kernels (dynamic): [Q^T fragments, where they are kept there][acc: kPaWaves x hp x D floats]
-// [m: kPaWaves x hp][l: kPaWaves x hp]; hp = query heads per pass of the cross-wave merge (chosen by the host so
-// that the whole fits 64 KiB).
+// LDS of the main kernels (dynamic): [Q^T fragments, where they are kept there][acc: kPaWaves x hp rows of
+// D + kPaAccPad floats][m: kPaWaves x hp][l: kPaWaves x hp]; hp = query heads per pass of the cross-wave merge
+// (chosen by the host so that the whole fits 64 KiB).  The pad keeps the rows of the 16 heads, which the lanes of
+// a wave write side by side, out of each other's banks.
+constexpr int kPaAccPad = 4;
+constexpr int kPaLdsPerHead(int head_dim) { return head_dim + kPaAccPad + 2; }  // floats per wave and head
 template <int D, int NSUB>
 constexpr bool pa_q_in_lds() { return PaDims<D>::kSlices * NSUB > 4; }
 template <int D, int NSUB>
@@ -283,7 +286,8 @@ __device__ __forceinline__ void pa_process_chunk(
   f16* sm_q = reinterpret_cast<f16*>(pa_lds);
   float* sm_acc = reinterpret_cast<float*>(pa_lds + pa_q_lds_halfs<D, NSUB>() * sizeof(f16));
   const int hp = ge.merge_heads;
-  float* sm_m = sm_acc + kPaWaves * hp * kPaD;
+  constexpr int kAccStride = kPaD + kPaAccPad;
+  float* sm_m = sm_acc + kPaWaves * hp * kAccStride;
   float* sm_l = sm_m + kPaWaves * hp;
 
   // Q^T operand: lane (head n of a sub-group, kg) holds q[head][32s + 8kg ..+7]; heads >= nh are zero
@@ -412,7 +416,7 @@ __device__ __forceinline__ void pa_process_chunk(
       const int cnt = min(hp, sub_end - h0);
       const int r = 16 * sg + n - h0;  // this lane's head inside the pass
       if (r >= 0 && r < cnt) {
-        float* dst = sm_acc + ((int64_t)(wave * hp + r)) * kPaD + 4 * kg;
+        float* dst = sm_acc + (wave * hp + r) * kAccStride + 4 * kg;
 #pragma unroll
         for (int db = 0; db < NOB; ++db) *reinterpret_cast<f32x4*>(dst + 16 * db) = st[sg].o[db];
         if (kg == 0) {
@@ -432,7 +436,7 @@ __device__ __forceinline__ void pa_process_chunk(
         for (int w = 0; w < kPaWaves; ++w) {
           const float wt = __builtin_amdgcn_exp2f(sm_m[w * hp + h] - mx);
           lsum += sm_l[w * hp + h] * wt;
-          a += sm_acc[(w * hp + h) * kPaD + d] * wt;
+          a += sm_acc[(w * hp + h) * kAccStride + d] * wt;
         }
         const int64_t head = (int64_t)b * num_heads + head0 + h0 + h;
         if (final) {
@@ -640,7 +644,7 @@ __global__ __launch_bounds__(kPaWaves* kWave) void pa_decode_balanced(
   if (planned) {
     extern __shared__ __attribute__((aligned(16))) unsigned char pa_lds[];
     int* plan_w = reinterpret_cast<int*>(pa_lds + pa_q_lds_halfs<D, NSUB>() * sizeof(f16)) +
-                  kPaWaves * ge.merge_heads * (D + 2);
+                  kPaWaves * ge.merge_heads * kPaLdsPerHead(D);
     pa_block_plan(context_lens, bs, max_len, (int)gridDim.x, w, plan_w, plan, w == 0 && blockIdx.y == 0);
     lds_plan = plan_w;
     total = lds_plan[2 * bs];
@@ -814,7 +818,7 @@ static int pa_subgroups(int64_t head_dim, int64_t group) {
 }
 
 static size_t pa_lds_bytes(int q_halfs, int merge_heads, int head_dim, int64_t bs, bool balanced) {
-  return (size_t)q_halfs * sizeof(f16) + (size_t)kPaWaves * merge_heads * (head_dim + 2) * sizeof(float) +
+  return (size_t)q_halfs * sizeof(f16) + (size_t)kPaWaves * merge_heads * kPaLdsPerHead(head_dim) * sizeof(float) +
          (balanced ? pa_block_plan_ints(bs) * sizeof(int) : 0);
 }
 
@@ -824,7 +828,7 @@ static int pa_merge_heads(int q_halfs, int head_dim, int heads, int64_t bs, bool
   const int sub = heads < kPaMaxGroup ? heads : kPaMaxGroup;
   const int64_t budget = 64 * 1024 - (int64_t)q_halfs * (int64_t)sizeof(f16) -
                          (int64_t)(balanced ? pa_block_plan_ints(bs) * sizeof(int) : 0);
-  int64_t cap = budget / (int64_t)(kPaWaves * (head_dim + 2) * sizeof(float));
+  int64_t cap = budget / (int64_t)(kPaWaves * kPaLdsPerHead(head_dim) * sizeof(float));
   if (cap < 1) cap = 1;
   if (cap > sub) cap = sub;
   const int passes = (int)((sub + cap - 1) / cap);

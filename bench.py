@@ -826,9 +826,13 @@ def bench_gmm_probe(L, R, dev):
     torch.manual_seed(0)
     gl = R.make_group_list(torch.randint(0, E, (rows,)), E).to(dev)
     out = []
-    for which, K, N in (("gate_up", hidden, 2 * inter), ("down", inter, hidden)):
+    gl_moe, rows_moe = gl, rows
+    for which, K, N in (("gate_up", hidden, 2 * inter), ("down", inter, hidden), ("dense", 8192, 8192)):
         g = torch.Generator(device=dev).manual_seed(1)
-        sets = 2
+        moe = which != "dense"   # the dense product: one group of 8192 rows (320-row tiles here, 256-row tiles in the "dense" line)
+        E, rows = (128, rows_moe) if moe else (1, 8192)
+        gl = gl_moe if moe else torch.tensor([rows], dtype=torch.int64, device=dev)
+        sets = 2 if moe else 1
         xs = [torch.randn(rows, K, generator=g, device=dev, dtype=torch.float16) for _ in range(sets)]
         ws = [torch.randn(E, N, K, generator=g, device=dev, dtype=torch.float16) * 0.02 for _ in range(sets)]
         ys = [torch.empty(rows, N, device=dev, dtype=torch.float16) for _ in range(sets)]
@@ -849,11 +853,16 @@ def bench_gmm_probe(L, R, dev):
         for parts_off, what in ((0, "whole kernel"), (9, "operand copies and barriers only"), (11, "weight copies only"),
                                 (13, "activation copies only"), (6, "MFMAs and LDS fragment reads only"), (14, "MFMAs only")):
             med, mn = timed(parts_off)
-            e = entry("grouped_matmul_probe", f"probe 4: MoE {which}, {what}", f"x [{rows},{K}] @ w [{E},{K},{N}] f16",
+            label = f"probe 4: MoE {which}" if moe else "probe dense 8192^3 (320-row tiles)"
+            e = entry("grouped_matmul_probe", f"{label}, {what}", f"x [{rows},{K}] @ w [{E},{K},{N}] f16",
                       "mfma", alg, flops, med, mn, None, None, 1,
                       None if parts_off == 0 else "parts of the k loop switched off: results wrong by construction, time only")
             e["parts_off"] = parts_off
             out.append(e)
+        if not moe:
+            del xs, ws, ys
+            torch.cuda.empty_cache()
+            continue
         # the same GEMM on weights whose rows are padded by one cache line (aops_grouped_matmul_ldw_f16): what the
         # power-of-two row stride of the reference's layout costs
         ldw = K + 64
