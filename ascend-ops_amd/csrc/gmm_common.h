@@ -304,7 +304,7 @@ int gmm_launch_persistent(bool swiglu, const f16* x, const f16* w, const int64_t
                           int64_t rows, int k, int num_experts, int n, hipStream_t stream,
                           const int32_t* row_idx, int idx_div, int64_t x_rows, int ldw = 0);
 int gmm_launch_persistent_probe(int parts_off, const f16* x, const f16* w, const int64_t* group_list, f16* y,
-                                int64_t rows, int k, int num_experts, int n, hipStream_t stream);
+                                int64_t rows, int k, int num_experts, int n, hipStream_t stream, int ldw);
 
 // Fused gate_up + SwiGLU (row_idx != nullptr: + row gather) on 128 x 128 tiles, or 64 x 64 with
 // `small`; k a multiple of 64.

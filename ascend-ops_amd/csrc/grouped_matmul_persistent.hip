@@ -558,11 +558,12 @@ int gmm_launch_persistent(bool swiglu, const f16* x, const f16* w, const int64_t
 
 // The 320 x 256 kernel with parts of its k loop switched off (see PROBE): a measurement aid.
 int gmm_launch_persistent_probe(int parts_off, const f16* x, const f16* w, const int64_t* group_list, f16* y,
-                                int64_t rows, int k, int num_experts, int n, hipStream_t stream) {
+                                int64_t rows, int k, int num_experts, int n, hipStream_t stream, int ldw) {
   switch (parts_off) {
-#define AOPS_PROBE_CASE(P) \
-  case (P):                \
-    return gmm_persistent_launch<5, 2, 4, false, false, (P)>(x, w, group_list, y, rows, k, num_experts, n, stream);
+#define AOPS_PROBE_CASE(P)                                                                                        \
+  case (P):                                                                                                       \
+    return gmm_persistent_launch<5, 2, 4, false, false, (P)>(x, w, group_list, y, rows, k, num_experts, n, stream, \
+                                                             nullptr, 1, 1, ldw);
     AOPS_PROBE_CASE(kProbeNoMfma | kProbeNoFragments)                       // 9: copies and barriers only
     AOPS_PROBE_CASE(kProbeNoMfma | kProbeNoFragments | kProbeNoXCopies)     // 11: weight copies only
     AOPS_PROBE_CASE(kProbeNoMfma | kProbeNoFragments | kProbeNoWCopies)     // 13: activation copies only

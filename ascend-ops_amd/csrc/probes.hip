@@ -5,30 +5,50 @@
 //    workgroup owns 128 consecutive rows of a [rows, row_bytes] byte matrix and walks along them in steps of
 //    seg_bytes per row - with seg_bytes = 128 and row_bytes = 2 * k that is how the weight tiles of the grouped
 //    matmul are fetched (128-byte pieces, one weight row apart); with row_bytes == seg_bytes the same kernel
-//    reads its 128 x seg_bytes block linearly.  No arithmetic beyond a sum that keeps the loads alive.
+//    reads its 128 x seg_bytes block linearly.  No arithmetic beyond a sum that keeps the loads alive.  The bytes
+//    go into registers or, like the operand copies of the persistent grouped-matmul kernel, straight into LDS.
 //  * aops_grouped_matmul_probe_f16: the persistent grouped-matmul kernel with parts of its k loop switched off.
 #include "gmm_common.h"
 
 namespace aops {
 
-template <int SEG>
+// VIA_LDS: the bytes are copied straight into LDS with global_load_lds_dwordx4, the instruction the persistent
+// grouped-matmul kernel fetches its operands with (a wave's 64 x 16 bytes land in 1 KiB of LDS that nobody reads),
+// instead of into registers.
+template <int SEG, bool VIA_LDS>
 __global__ __launch_bounds__(256) void probe_read_stream_kernel(const char* __restrict__ buf, float* __restrict__ sink,
                                                                 int64_t row_bytes) {
   constexpr int kLanesPerRow = SEG / 16;
   constexpr int kRowsPerPass = 256 / kLanesPerRow;
   constexpr int kPasses = 128 / kRowsPerPass;
+  __shared__ __attribute__((aligned(16))) char landing[VIA_LDS ? 4 * kPasses * 1024 : 16];
   const char* base = buf + (int64_t)blockIdx.x * 128 * row_bytes;
   const int r0 = threadIdx.x / kLanesPerRow;
   const int c = threadIdx.x % kLanesPerRow;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int64_t off = 0; off < row_bytes; off += SEG) {
-    f32x4 v[kPasses];
+  if constexpr (VIA_LDS) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)AOPS_LDS_PTR(landing) + (uint32_t)wave * kPasses * 1024u;
+    for (int64_t off = 0; off < row_bytes; off += SEG) {
 #pragma unroll
-    for (int p = 0; p < kPasses; ++p)
-      v[p] = __builtin_nontemporal_load(
-          reinterpret_cast<const f32x4*>(base + (int64_t)(r0 + p * kRowsPerPass) * row_bytes + off + c * 16));
+      for (int p = 0; p < kPasses; ++p) {
+        const char* src = base + (int64_t)(r0 + p * kRowsPerPass) * row_bytes + off + c * 16;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                     :: "s"(lds0 + p * 1024u), "v"(src) : "memory");
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next step reuses the landing area
+    }
+    acc[0] = (float)landing[threadIdx.x & 15];
+  } else {
+    for (int64_t off = 0; off < row_bytes; off += SEG) {
+      f32x4 v[kPasses];
 #pragma unroll
-    for (int p = 0; p < kPasses; ++p) acc += v[p];
+      for (int p = 0; p < kPasses; ++p)
+        v[p] = __builtin_nontemporal_load(
+            reinterpret_cast<const f32x4*>(base + (int64_t)(r0 + p * kRowsPerPass) * row_bytes + off + c * 16));
+#pragma unroll
+      for (int p = 0; p < kPasses; ++p) acc += v[p];
+    }
   }
   // never true for the buffers the probe is run on (finite values): the store only keeps the loads alive
   if (acc[0] + acc[1] + acc[2] + acc[3] == 12345.678f) sink[0] = acc[0];
@@ -37,43 +57,44 @@ __global__ __launch_bounds__(256) void probe_read_stream_kernel(const char* __re
 }  // namespace aops
 
 extern "C" int aops_probe_read_stream(const void* buf, int64_t rows, int64_t row_bytes, int64_t seg_bytes,
-                                      void* sink, void* stream) {
+                                      int via_lds, void* sink, void* stream) {
   using namespace aops;
   if (rows <= 0 || rows % 128 != 0 || rows / 128 > 0x7fffffff || row_bytes <= 0 || !buf || !sink)
     return AOPS_ERR_INVALID_ARGUMENT;
   if ((seg_bytes != 128 && seg_bytes != 256 && seg_bytes != 512 && seg_bytes != 1024) || row_bytes % seg_bytes != 0)
     return AOPS_ERR_INVALID_ARGUMENT;
+  if (via_lds != 0 && via_lds != 1) return AOPS_ERR_INVALID_ARGUMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const unsigned grid = (unsigned)(rows / 128);
   const char* p = static_cast<const char*>(buf);
   float* out = static_cast<float*>(sink);
+#define AOPS_STREAM_CASE(SEG)                                                               \
+  case SEG:                                                                                 \
+    if (via_lds)                                                                            \
+      probe_read_stream_kernel<SEG, true><<<grid, 256, 0, s>>>(p, out, row_bytes);          \
+    else                                                                                    \
+      probe_read_stream_kernel<SEG, false><<<grid, 256, 0, s>>>(p, out, row_bytes);         \
+    break;
   switch (seg_bytes) {
-    case 128:
-      probe_read_stream_kernel<128><<<grid, 256, 0, s>>>(p, out, row_bytes);
-      break;
-    case 256:
-      probe_read_stream_kernel<256><<<grid, 256, 0, s>>>(p, out, row_bytes);
-      break;
-    case 512:
-      probe_read_stream_kernel<512><<<grid, 256, 0, s>>>(p, out, row_bytes);
-      break;
-    default:
-      probe_read_stream_kernel<1024><<<grid, 256, 0, s>>>(p, out, row_bytes);
-      break;
+    AOPS_STREAM_CASE(128)
+    AOPS_STREAM_CASE(256)
+    AOPS_STREAM_CASE(512)
+    AOPS_STREAM_CASE(1024)
   }
+#undef AOPS_STREAM_CASE
   return record_launch_status(hipGetLastError());
 }
 
-extern "C" int aops_grouped_matmul_probe_f16(int parts_off, const void* x, const void* w,
+extern "C" int aops_grouped_matmul_probe_f16(int parts_off, const void* x, const void* w, int64_t ldw,
                                              const int64_t* group_list, void* y, int64_t rows, int64_t k,
                                              int64_t num_experts, int64_t n, void* stream) {
   using namespace aops;
   // the shapes the persistent 320 x 256 kernel takes
-  if (rows <= 0 || num_experts <= 0 || k < 256 || k % 128 != 0 || k > (1 << 22) || n <= 0 || n % 64 != 0 ||
-      rows > 0x7fffffff - 4096 || n > 0x7fffffff || num_experts > (1 << 20))
+  if (rows <= 0 || num_experts <= 0 || k < 256 || k % 128 != 0 || ldw < k || ldw % 8 != 0 || ldw > (1 << 22) || n <= 0 ||
+      n % 64 != 0 || rows > 0x7fffffff - 4096 || n > 0x7fffffff || num_experts > (1 << 20))
     return AOPS_ERR_INVALID_ARGUMENT;
   if (!x || !w || !y || (!group_list && num_experts != 1)) return AOPS_ERR_INVALID_ARGUMENT;
   return gmm_launch_persistent_probe(parts_off, static_cast<const f16*>(x), static_cast<const f16*>(w), group_list,
                                      static_cast<f16*>(y), rows, (int)k, (int)num_experts, (int)n,
-                                     static_cast<hipStream_t>(stream));
+                                     static_cast<hipStream_t>(stream), (int)ldw);
 }

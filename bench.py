@@ -570,13 +570,47 @@ def bench_moe_one(L, ops, R, dev, which):
     torch.manual_seed(0)
     rows = tokens * topk
     gl = R.make_group_list(torch.randint(0, E, (rows,)), E)
-    K, N = (hidden, 2 * inter) if which == "gate_up" else (inter, hidden)
-    x = (torch.randn(rows, K) * (1.0 if which == "gate_up" else 0.3)).half()
+    K, N = (hidden, 2 * inter) if which.startswith("gate_up") else (inter, hidden)
+    x = (torch.randn(rows, K) * (1.0 if which.startswith("gate_up") else 0.3)).half()
     w = torch.empty(E, N, K, dtype=torch.float16)
     for e in range(E):
         w[e] = (0.02 * torch.randn(N, K)).half()
+    if which.endswith("_padded"):
+        return _gmm_padded_entry(L, dev, which, x, w, gl)
     e, _ = _gmm_entry(L, ops, R, dev, False, "grouped_matmul", f"4: MoE {which} (alone)", x, w, gl)
     return e
+
+
+def _gmm_padded_entry(L, dev, which, x, w, gl):
+    """One GEMM of configs[3] over weights whose rows are padded by one cache line (aops_grouped_matmul_ldw_f16), alone in
+    its run so that a profiler can tell it from the unpadded launches; checked bit for bit against the unpadded kernel."""
+    import torch
+
+    rows, K = x.shape
+    E, N, _ = w.shape
+    ldw = K + 64
+    xd, wd, gd = x.to(dev), w.to(dev), gl.to(dev)
+    y_ref = torch.empty(rows, N, dtype=torch.float16, device=dev)
+    L.check(L.lib.aops_grouped_matmul_variant_f16(6, xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y_ref.data_ptr(), rows, K,
+                                                  E, N, L.stream()))
+    sets = 2
+    wps = []
+    for _ in range(sets):
+        wp = torch.zeros(E, N, ldw, dtype=torch.float16, device=dev)
+        wp[:, :, :K] = wd
+        wps.append(wp)
+    del wd
+    xs = [xd, xd.clone()]
+    ys = [torch.empty(rows, N, dtype=torch.float16, device=dev) for _ in range(sets)]
+    calls = [(lambda i=i: L.check(L.lib.aops_grouped_matmul_ldw_f16(xs[i].data_ptr(), wps[i].data_ptr(), ldw, gd.data_ptr(),
+                                                                    ys[i].data_ptr(), rows, K, E, N, L.stream())))
+             for i in range(sets)]
+    med, mn = time_graph(calls, min_launches=40)
+    assert torch.equal(ys[0], y_ref), "padded weight rows must give the same bits"
+    end = int(gl[-1])
+    return entry("grouped_matmul_ldw", f"4: MoE {which} (alone; weight rows {2 * ldw} bytes apart)",
+                 f"x [{rows},{K}] @ w [{E},{K},{N}] f16", "mfma", rows * K * 2 + E * N * K * 2 + end * N * 2 + E * 8,
+                 2 * end * K * N, med, mn, None, None, 1)
 
 
 def bench_mlp(L, ops, R, dev, cpu):
@@ -839,15 +873,15 @@ def bench_gmm_probe(L, R, dev):
         flops = 2 * rows * K * N
         alg = rows * K * 2 + E * N * K * 2 + rows * N * 2 + E * 8
 
-        def timed(parts_off):
+        def timed(parts_off, wsrc=None, ld=None):
             if parts_off == 0:
                 calls = [(lambda i=i: L.check(L.lib.aops_grouped_matmul_variant_f16(
                     6, xs[i].data_ptr(), ws[i].data_ptr(), gl.data_ptr(), ys[i].data_ptr(), rows, K, E, N, L.stream())))
                     for i in range(sets)]
             else:
                 calls = [(lambda i=i: L.check(L.lib.aops_grouped_matmul_probe_f16(
-                    parts_off, xs[i].data_ptr(), ws[i].data_ptr(), gl.data_ptr(), ys[i].data_ptr(), rows, K, E, N,
-                    L.stream()))) for i in range(sets)]
+                    parts_off, xs[i].data_ptr(), (wsrc or ws)[i].data_ptr(), ld or K, gl.data_ptr(), ys[i].data_ptr(), rows, K,
+                    E, N, L.stream()))) for i in range(sets)]
             return time_graph(calls, min_launches=40, trials=3)
 
         for parts_off, what in ((0, "whole kernel"), (9, "operand copies and barriers only"), (11, "weight copies only"),
@@ -884,19 +918,30 @@ def bench_gmm_probe(L, R, dev):
         out.append(entry("grouped_matmul_ldw", f"probe 4: MoE {which}, weight rows padded to {2 * ldw} bytes (extension)",
                          f"x [{rows},{K}] @ w [{E},{K},{N}] f16, row stride {ldw}", "mfma", alg, flops, med, mn, None, None, 1,
                          "same kernel and same bits as the whole-kernel line; the caller pads the static weights once"))
+        for parts_off, what in ((9, "operand copies and barriers only"), (11, "weight copies only")):
+            med, mn = timed(parts_off, wps, ldw)
+            e = entry("grouped_matmul_probe", f"probe 4: MoE {which}, weight rows padded to {2 * ldw} bytes, {what}",
+                      f"x [{rows},{K}] @ w [{E},{K},{N}] f16, row stride {ldw}", "mfma", alg, flops, med, mn, None, None, 1,
+                      "parts of the k loop switched off: results wrong by construction, time only")
+            e["parts_off"] = parts_off
+            out.append(e)
         del wps, y_pad
         # the weight bytes of this GEMM as a pure read stream: the kernel's pattern, longer pieces, and linear
         wbytes = E * N * K * 2
         sink = torch.zeros(1, dtype=torch.float32, device=dev)
-        for seg, row_bytes, what in ((128, 2 * K, f"128-byte pieces one weight row ({2 * K} B) apart, as the kernel copies them"),
-                                     (256, 2 * K, "256-byte pieces one weight row apart"),
-                                     (512, 2 * K, "512-byte pieces one weight row apart"),
-                                     (128, 2 * K + 128, f"128-byte pieces {2 * K + 128} B apart (what a row padded by one line would give)"),
-                                     (1024, 1024, "the same bytes read linearly (1 KiB per row of the probe)")):
+        for seg, row_bytes, via_lds, what in (
+                (128, 2 * K, 0, f"128-byte pieces one weight row ({2 * K} B) apart, as the kernel copies them"),
+                (256, 2 * K, 0, "256-byte pieces one weight row apart"),
+                (512, 2 * K, 0, "512-byte pieces one weight row apart"),
+                (128, 2 * K + 128, 0, f"128-byte pieces {2 * K + 128} B apart (what a row padded by one line would give)"),
+                (1024, 1024, 0, "the same bytes read linearly (1 KiB per row of the probe)"),
+                (128, 2 * K, 1, f"128-byte pieces {2 * K} B apart, copied straight into LDS (the kernel's copy instruction)"),
+                (128, 2 * K + 128, 1, f"128-byte pieces {2 * K + 128} B apart, copied straight into LDS"),
+                (1024, 1024, 1, "read linearly, copied straight into LDS")):
             if row_bytes % seg != 0:
                 continue
             nrows = wbytes // row_bytes // 128 * 128
-            calls = [(lambda i=i: L.check(L.lib.aops_probe_read_stream(ws[i].data_ptr(), nrows, row_bytes, seg,
+            calls = [(lambda i=i: L.check(L.lib.aops_probe_read_stream(ws[i].data_ptr(), nrows, row_bytes, seg, via_lds,
                                                                         sink.data_ptr(), L.stream()))) for i in range(sets)]
             med, mn = time_graph(calls, min_launches=40, trials=3)
             out.append(entry("read_stream_probe", f"probe 4: weights of MoE {which} as a read stream, {what}",
@@ -994,6 +1039,7 @@ def main():
     if args.skip_headline:
         for tag, fn in (("moe_gate_up", lambda: bench_moe_one(L, ops, R, dev, "gate_up")),
                         ("moe_down", lambda: bench_moe_one(L, ops, R, dev, "down")),
+                        ("moe_gate_up_padded", lambda: bench_moe_one(L, ops, R, dev, "gate_up_padded")),
                         ("dense", lambda: bench_dense(L, R, dev)),
                         ("gmm_probe", lambda: bench_gmm_probe(L, R, dev)),
                         ("pa_more", lambda: bench_pa_more(L, R, dev, cpu))):

@@ -343,24 +343,28 @@ int aops_empty_launch(int64_t workgroups, int threads, void* stream);
  * [rows, row_bytes] byte matrix (rows a multiple of 128); every workgroup owns 128 consecutive rows and
  * walks along them in steps of seg_bytes (128, 256, 512 or 1024, dividing row_bytes) per row.  With
  * seg_bytes = 128 and row_bytes = 2 * k this is how the weight tiles of the grouped matmul are fetched;
- * with row_bytes == seg_bytes every workgroup reads one contiguous block (a linear stream).  sink: 4 bytes
- * of device memory that are never written for finite data.  Bandwidth = rows * row_bytes / duration.
+ * with row_bytes == seg_bytes every workgroup reads one contiguous block (a linear stream).  via_lds: 0 =
+ * ordinary 128-bit loads into registers, 1 = global_load_lds_dwordx4 straight into LDS, the instruction the
+ * persistent grouped-matmul kernel fetches its operands with.  sink: 4 bytes of device memory that are never
+ * written for finite data.  Bandwidth = rows * row_bytes / duration.
  * No counterpart in the reference.
  */
-int aops_probe_read_stream(const void* buf, int64_t rows, int64_t row_bytes, int64_t seg_bytes, void* sink,
-                           void* stream);
+int aops_probe_read_stream(const void* buf, int64_t rows, int64_t row_bytes, int64_t seg_bytes, int via_lds,
+                           void* sink, void* stream);
 
 /*
  * Measurement aid: the persistent 320 x 256 kernel of aops_grouped_matmul_f16 (k % 128 == 0, k >= 256)
- * with parts of its k loop switched off, to time what the rest costs by itself.  parts_off: 9 = operand
+ * with parts of its k loop switched off, to time what the rest costs by itself.  ldw = elements from one
+ * weight row to the next (k: densely packed, as the operator takes them; more: padded rows, as
+ * aops_grouped_matmul_ldw_f16 takes them).  parts_off: 9 = operand
  * copies and barriers only (no MFMAs, no LDS fragment reads), 11 = weight copies only, 13 = activation
  * copies only, 6 = MFMAs and fragment reads only (no copies), 14 = MFMAs only; anything else returns
  * AOPS_ERR_INVALID_ARGUMENT.  y is written with values that are wrong by construction.
  * No counterpart in the reference.
  */
-int aops_grouped_matmul_probe_f16(int parts_off, const void* x, const void* w, const int64_t* group_list,
-                                  void* y, int64_t rows, int64_t k, int64_t num_experts, int64_t n,
-                                  void* stream);
+int aops_grouped_matmul_probe_f16(int parts_off, const void* x, const void* w, int64_t ldw,
+                                  const int64_t* group_list, void* y, int64_t rows, int64_t k, int64_t num_experts,
+                                  int64_t n, void* stream);
 
 /*
  * Device summary (CU count, LDS, L2, memory size, clocks) written as text into buf

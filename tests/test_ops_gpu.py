@@ -381,25 +381,29 @@ def test_measurement_aids_run_and_leave_their_surroundings_alone(dev):
     xd, wd, gd = x.to(dev), w.transpose(1, 2).contiguous().to(dev), gl.to(dev)
     y = torch.full((rows + 2, N), 7.0, dtype=H, device=dev)        # one guard row on either side
     for parts_off in (9, 11, 13, 6, 14):
-        assert lib.aops_grouped_matmul_probe_f16(parts_off, xd.data_ptr(), wd.data_ptr(), gd.data_ptr(),
+        assert lib.aops_grouped_matmul_probe_f16(parts_off, xd.data_ptr(), wd.data_ptr(), K, gd.data_ptr(),
                                                  y[1:].data_ptr(), rows, K, E, N, cabi.stream(dev)) == 0
     torch.cuda.synchronize()
     assert torch.all(y[0] == 7.0) and torch.all(y[-1] == 7.0)
     for bad in (0, 1, 7, 15, -1):
-        assert lib.aops_grouped_matmul_probe_f16(bad, xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y[1:].data_ptr(),
+        assert lib.aops_grouped_matmul_probe_f16(bad, xd.data_ptr(), wd.data_ptr(), K, gd.data_ptr(), y[1:].data_ptr(),
                                                  rows, K, E, N, cabi.stream(dev)) == -1
-    assert lib.aops_grouped_matmul_probe_f16(9, xd.data_ptr(), wd.data_ptr(), gd.data_ptr(), y[1:].data_ptr(),
+    assert lib.aops_grouped_matmul_probe_f16(9, xd.data_ptr(), wd.data_ptr(), 192, gd.data_ptr(), y[1:].data_ptr(),
                                              rows, 192, E, N, cabi.stream(dev)) == -1    # k the kernel does not take
+    assert lib.aops_grouped_matmul_probe_f16(9, xd.data_ptr(), wd.data_ptr(), K - 8, gd.data_ptr(), y[1:].data_ptr(),
+                                             rows, K, E, N, cabi.stream(dev)) == -1      # row stride below k
     buf = torch.ones(256 * 1024, dtype=torch.uint8, device=dev)
     sink = torch.zeros(1, dtype=torch.float32, device=dev)
-    for seg, row_bytes in ((128, 1024), (256, 512), (512, 512), (1024, 1024), (128, 128)):
-        assert lib.aops_probe_read_stream(buf.data_ptr(), buf.numel() // row_bytes, row_bytes, seg, sink.data_ptr(),
-                                          cabi.stream(dev)) == 0
+    for via_lds in (0, 1):
+        for seg, row_bytes in ((128, 1024), (256, 512), (512, 512), (1024, 1024), (128, 128)):
+            assert lib.aops_probe_read_stream(buf.data_ptr(), buf.numel() // row_bytes, row_bytes, seg, via_lds,
+                                              sink.data_ptr(), cabi.stream(dev)) == 0
     torch.cuda.synchronize()
     assert float(sink[0]) == 0.0
-    assert lib.aops_probe_read_stream(buf.data_ptr(), 100, 1024, 128, sink.data_ptr(), cabi.stream(dev)) == -1   # rows % 128
-    assert lib.aops_probe_read_stream(buf.data_ptr(), 256, 1024, 96, sink.data_ptr(), cabi.stream(dev)) == -1    # piece size
-    assert lib.aops_probe_read_stream(buf.data_ptr(), 256, 640, 256, sink.data_ptr(), cabi.stream(dev)) == -1    # not dividing
+    assert lib.aops_probe_read_stream(buf.data_ptr(), 100, 1024, 128, 0, sink.data_ptr(), cabi.stream(dev)) == -1   # rows % 128
+    assert lib.aops_probe_read_stream(buf.data_ptr(), 256, 1024, 96, 0, sink.data_ptr(), cabi.stream(dev)) == -1    # piece size
+    assert lib.aops_probe_read_stream(buf.data_ptr(), 256, 640, 256, 0, sink.data_ptr(), cabi.stream(dev)) == -1    # not dividing
+    assert lib.aops_probe_read_stream(buf.data_ptr(), 256, 1024, 128, 2, sink.data_ptr(), cabi.stream(dev)) == -1   # via_lds
 
 
 @pytest.mark.parametrize("seed", range(12))
