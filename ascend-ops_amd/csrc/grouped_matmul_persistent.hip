@@ -569,6 +569,8 @@ int gmm_launch_persistent_probe(int parts_off, const f16* x, const f16* w, const
     AOPS_PROBE_CASE(kProbeNoMfma | kProbeNoFragments | kProbeNoWCopies)     // 13: activation copies only
     AOPS_PROBE_CASE(kProbeNoXCopies | kProbeNoWCopies)                      // 6: MFMAs and fragment reads only
     AOPS_PROBE_CASE(kProbeNoXCopies | kProbeNoWCopies | kProbeNoFragments)  // 14: MFMAs only
+    AOPS_PROBE_CASE(kProbeNoMfma)                                           // 1: copies and LDS fragment reads, no MFMAs
+    AOPS_PROBE_CASE(kProbeNoFragments)                                      // 8: copies and MFMAs, no LDS fragment reads
 #undef AOPS_PROBE_CASE
     default:
       return AOPS_ERR_INVALID_ARGUMENT;

@@ -885,7 +885,8 @@ def bench_gmm_probe(L, R, dev):
             return time_graph(calls, min_launches=40, trials=3)
 
         for parts_off, what in ((0, "whole kernel"), (9, "operand copies and barriers only"), (11, "weight copies only"),
-                                (13, "activation copies only"), (6, "MFMAs and LDS fragment reads only"), (14, "MFMAs only")):
+                                (13, "activation copies only"), (6, "MFMAs and LDS fragment reads only"), (14, "MFMAs only"),
+                                (1, "copies and LDS fragment reads, no MFMAs"), (8, "copies and MFMAs, no LDS fragment reads")):
             med, mn = timed(parts_off)
             label = f"probe 4: MoE {which}" if moe else "probe dense 8192^3 (320-row tiles)"
             e = entry("grouped_matmul_probe", f"{label}, {what}", f"x [{rows},{K}] @ w [{E},{K},{N}] f16",

@@ -358,7 +358,8 @@ int aops_probe_read_stream(const void* buf, int64_t rows, int64_t row_bytes, int
  * weight row to the next (k: densely packed, as the operator takes them; more: padded rows, as
  * aops_grouped_matmul_ldw_f16 takes them).  parts_off: 9 = operand
  * copies and barriers only (no MFMAs, no LDS fragment reads), 11 = weight copies only, 13 = activation
- * copies only, 6 = MFMAs and fragment reads only (no copies), 14 = MFMAs only; anything else returns
+ * copies only, 6 = MFMAs and fragment reads only (no copies), 14 = MFMAs only, 1 = everything but the MFMAs,
+ * 8 = everything but the LDS fragment reads; anything else returns
  * AOPS_ERR_INVALID_ARGUMENT.  y is written with values that are wrong by construction.
  * No counterpart in the reference.
  */
