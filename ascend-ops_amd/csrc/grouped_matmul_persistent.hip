@@ -67,8 +67,12 @@ constexpr int kEpiScratchHalfs = 512;         // 1 KiB of LDS per wave for the e
 
 // PROBE (measurement aid, results wrong by construction): parts of the k loop switched off, so that what
 // the rest costs by itself can be timed: bit 0 = no MFMAs, bit 1 = no activation copies, bit 2 = no weight
-// copies, bit 3 = no LDS fragment reads (the MFMAs then run on registers that never change).  0 = the kernel.
-constexpr int kProbeNoMfma = 1, kProbeNoXCopies = 2, kProbeNoWCopies = 4, kProbeNoFragments = 8;
+// copies, bit 3 = no LDS fragment reads (the MFMAs then run on registers that never change), bit 4 = the weight
+// copies of a k tile fetch 256 bytes of every row of one half of the tile's rows (even tiles the first half, odd
+// tiles the second, both at the even tile's k offset) instead of 128 bytes of every row: the same requests per
+// tile and the same bytes per pair of tiles, in pieces twice as long; where they land in LDS is meaningless, so
+// only together with bits 0 and 3.  0 = the kernel.
+constexpr int kProbeNoMfma = 1, kProbeNoXCopies = 2, kProbeNoWCopies = 4, kProbeNoFragments = 8, kProbeWidePieces = 16;
 
 template <int MB, int NB, int WN, bool SWIGLU, bool GATHER, int PROBE = 0>
 __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kernel(
@@ -161,6 +165,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   const uint32_t off0_w = ((uint32_t)lane_row * (uint32_t)ldw + lane_c * 8) * 2u;
   const uint32_t copy_stride_w = 8u * kWaves * (uint32_t)ldw * 2u;
   uint32_t a_last, b_last;  // offset of this lane's chunk in the last valid row
+  uint32_t b_rows = 1;      // valid weight rows of the item (used by the wide-piece measurement build only)
   uint32_t a_src[GATHER ? kACopies : 1];  // GATHER: offset of this lane's chunk per copy
   // SWIGLU: copy i of the weights fills row blocks 2i (gate rows 32i..32i+31 of the item) and
   // 2i+1 (the up rows d further down): per-lane offset + 32 rows per copy; b_last then holds the
@@ -173,6 +178,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     b_base = w + ((int64_t)it.expert * n + (int64_t)it.n_tile * BNO) * ldw;
     const int n_left = min(n_out - it.n_tile * BNO, BNO);
     b_last = SWIGLU ? (uint32_t)(n_left / 32) : ((uint32_t)(n_left - 1) * (uint32_t)ldw + lane_c * 8) * 2u;
+    b_rows = (uint32_t)n_left;
   };
   auto set_x_sources = [&](const GmmWork& it) {
     const int lane_s = lane_id_fresh();
@@ -203,27 +209,39 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   };
   const uint32_t lds_sa = (uint32_t)(uintptr_t)AOPS_LDS_PTR(sa);  // LDS byte addresses of the stages
   const uint32_t lds_sb = (uint32_t)(uintptr_t)AOPS_LDS_PTR(sb);
-  auto copy_x = [&](int kt, int stage) {
+  // copy i of the activation tile kt into its stage (kACopies per wave and tile), copy i of the weight tile
+  auto copy_x_one = [&](int kt, int stage, int i) {
     if constexpr (PROBE & kProbeNoXCopies) return;
     const int ko = kt * kBK;
     const uint32_t da = lds_sa + (uint32_t)(stage * BM * kBK + wave * 512) * 2u;
-#pragma unroll
-    for (int i = 0; i < kACopies; ++i) {
-      if constexpr (GATHER) {  // offsets of up to 2^32 elements: 64-bit address per lane
-        dma16(a_base + ko + a_src[i], da + i * kWaves * 1024);
-      } else {
-        // uniform base + 32-bit byte offset per lane: the copy takes them as they are (scalar base,
-        // vector offset), no vector instructions spent on a 64-bit address
-        dma16(a_base + ko, min(off0 + i * copy_stride, a_last), da + i * kWaves * 1024);
-      }
+    if constexpr (GATHER) {  // offsets of up to 2^32 elements: 64-bit address per lane
+      dma16(a_base + ko + a_src[i], da + i * kWaves * 1024);
+    } else {
+      // uniform base + 32-bit byte offset per lane: the copy takes them as they are (scalar base,
+      // vector offset), no vector instructions spent on a 64-bit address
+      dma16(a_base + ko, min(off0 + i * copy_stride, a_last), da + i * kWaves * 1024);
     }
   };
-  auto copy_w = [&](int kt, int stage) {
+  auto copy_x = [&](int kt, int stage) {
+#pragma unroll
+    for (int i = 0; i < kACopies; ++i) copy_x_one(kt, stage, i);
+  };
+  auto copy_w_one = [&](int kt, int stage, int i) {
     if constexpr (PROBE & kProbeNoWCopies) return;
     const int ko = kt * kBK;
     const uint32_t db = lds_sb + (uint32_t)(stage * BN * kBK + wave * 512) * 2u;
+    if constexpr (PROBE & kProbeWidePieces) {
+      static_assert(!(PROBE & kProbeWidePieces) || (!SWIGLU && BN == 256 && kBCopies * kWaves * 4 == 128), "half a tile per copy round");
+      const int lane_s = lane_id_fresh();  // a copy = 4 rows x 256 bytes
+      const uint32_t row = min((uint32_t)((kt & 1) * 128 + (i * kWaves + wave) * 4 + (lane_s >> 4)), b_rows - 1u);
+      dma16(b_base + (kt & ~1) * kBK, (row * (uint32_t)ldw + (uint32_t)(lane_s & 15) * 8u) * 2u, db + i * kWaves * 1024);
+      return;
+    }
+    dma16(b_base + ko, b_offset(i), db + i * kWaves * 1024);
+  };
+  auto copy_w = [&](int kt, int stage) {
 #pragma unroll
-    for (int i = 0; i < kBCopies; ++i) dma16(b_base + ko, b_offset(i), db + i * kWaves * 1024);
+    for (int i = 0; i < kBCopies; ++i) copy_w_one(kt, stage, i);
   };
 
   const int fm = lane & 31;
@@ -245,16 +263,17 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   // registers at once and its activation fragments one at a time, row block by row block:
   //
   //   barrier A(t): tile t has landed, nobody reads the activation stage of tile t-1 any more
-  //     -> activation copies of tile t+1, fragment reads of tile t between the last eight MFMAs of tile t-1
+  //     -> fragment reads of tile t between the last eight MFMAs of tile t-1, first MFMAs of tile t; the
+  //        activation copies of tile t+1 one at a time between them
   //   barrier B(t): everybody holds the weight fragments of tile t in registers
-  //     -> weight copies of tile t+2 into the weight stage of tile t
-  //   MFMAs of tile t ...
+  //     -> the other MFMAs of tile t; the weight copies of tile t+2 (into the weight stage of tile t) one at a
+  //        time between them
   //
   // The weights are read once, so each of their requests goes to memory and is slow; the activation
   // rows mostly hit in L2.  Freeing the weight stage at the start of the tile gives the slow requests
-  // almost two tile periods to arrive, and barrier A(t+1) waits only for copies that were issued a full
-  // period before: the L1's queue of pending requests (what bounds this kernel) still holds the weight
-  // requests of tile t+2 when the next burst arrives, instead of draining to empty at every barrier.
+  // more than a tile period to arrive, and barrier A(t+1) waits only for copies that were issued most of a
+  // period before: the L1's queue of pending requests (what bounds this kernel) still holds requests of
+  // tile t+2 when the next ones arrive, instead of draining to empty at every barrier.
   auto k_loop = [&](auto live_c) {
     constexpr int LIVE = decltype(live_c)::value;
     constexpr int NF = kSteps * LIVE;  // activation fragments (pairs of MFMAs) of a k tile
@@ -306,14 +325,16 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
       asm volatile("" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
     };
-    // MFMA pairs N .. END-1 of the tile, each followed by the read of the fragment that takes its place
-    auto pairs = [&](auto self, auto n_c, auto end_c, auto stage_c) {
+    // MFMA pairs N .. END-1 of the tile, each followed by the copies that hook(N) issues and by the read of the
+    // fragment that takes the pair's place
+    auto pairs = [&](auto self, auto n_c, auto end_c, auto stage_c, auto&& hook) {
       constexpr int N = decltype(n_c)::value;
       if constexpr (N < decltype(end_c)::value) {
         mma(n_c);
+        hook(n_c);
         read_fa(std::integral_constant<int, N + kFa>{}, stage_c);
         __builtin_amdgcn_sched_barrier(0);
-        self(self, std::integral_constant<int, N + 1>{}, end_c, stage_c);
+        self(self, std::integral_constant<int, N + 1>{}, end_c, stage_c, hook);
       }
     };
     // The last kTail pairs of a tile run at the start of the next one, between its first fragment reads,
@@ -322,14 +343,33 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     // barrier B comes after this many pairs of the tile: the burst of reads at its start has returned by
     // then, so the wait in front of the barrier costs nothing
     constexpr int kPairsBeforeB = NF - kTail < 6 ? NF - kTail : 6;
+    // The copies of a tile are spread over the MFMA pairs between its barriers instead of following the
+    // barrier in one burst: a copy cannot issue while the L1's queue of pending requests is full, a wave
+    // stuck at a copy issues no MFMAs, and a burst of four or five copies from each of the eight waves is
+    // several queues long - while the queue, once the burst is in, drains with nothing behind it until the
+    // next barrier.  One copy every other pair keeps the queue fed at the rate it empties and costs a wave
+    // a few lines' worth of waiting at a time, which the MFMAs in flight cover.
+    constexpr int kSlotsA = LIVE > 0 ? kTail + kPairsBeforeB : 0;  // tail pairs + pairs between barrier A and barrier B
+    constexpr int kSlotsB = NF - kTail - kPairsBeforeB;            // pairs between barrier B and the next barrier A
     auto tile = [&](auto stage_c, int kx, int kw, bool tail, bool switch_x, bool switch_w) {
       constexpr int STAGE = decltype(stage_c)::value;
       if (switch_x) set_x_sources(nxt);
-      copy_x(kx, STAGE ^ 1);
+      auto x_copies_of_slot = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < kACopies; ++i)
+          if (kSlotsA > 0 && i * kSlotsA / kACopies == slot) copy_x_one(kx, STAGE ^ 1, i);
+      };
+      auto w_copies_of_slot = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < kBCopies; ++i)
+          if (kSlotsB > 0 && i * kSlotsB / kBCopies == slot) copy_w_one(kw, STAGE, i);
+      };
+      if constexpr (kSlotsA == 0) copy_x(kx, STAGE ^ 1);
       if constexpr (LIVE > 0) {
         auto start = [&](auto q_c) {  // tail pair q of the previous tile, then the reads that reuse its registers
           constexpr int Q = decltype(q_c)::value;
           if (tail) mma(std::integral_constant<int, NF - kTail + Q>{});
+          x_copies_of_slot(Q);
           read_fa(q_c, stage_c);
           __builtin_amdgcn_sched_barrier(0);  // the counted wait in front of barrier B relies on this order
           read_fb(q_c, stage_c);
@@ -339,7 +379,8 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
         start(std::integral_constant<int, 1>{});
         start(std::integral_constant<int, 2>{});
         start(std::integral_constant<int, 3>{});
-        pairs(pairs, std::integral_constant<int, 0>{}, std::integral_constant<int, kPairsBeforeB>{}, stage_c);
+        pairs(pairs, std::integral_constant<int, 0>{}, std::integral_constant<int, kPairsBeforeB>{}, stage_c,
+              [&](auto n_c) { x_copies_of_slot(kTail + decltype(n_c)::value); });
       }
       // all own weight fragments of this tile are in registers (LDS serves a wave's reads in order, and only
       // the kPairsBeforeB refills of the activation ring were issued after the last of them) ...
@@ -349,9 +390,10 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
       __builtin_amdgcn_s_barrier();  // ... and so are everybody else's: barrier B
       fence();
       if (switch_w) set_w_sources(nxt);
-      copy_w(kw, STAGE);
+      if constexpr (kSlotsB == 0) copy_w(kw, STAGE);
       if constexpr (LIVE > 0)
-        pairs(pairs, std::integral_constant<int, kPairsBeforeB>{}, std::integral_constant<int, NF - kTail>{}, stage_c);
+        pairs(pairs, std::integral_constant<int, kPairsBeforeB>{}, std::integral_constant<int, NF - kTail>{}, stage_c,
+              [&](auto n_c) { w_copies_of_slot(decltype(n_c)::value - kPairsBeforeB); });
       // own copies of the next tile (all but the weight copies just issued) and all own fragment reads of
       // this tile are complete ...
       __builtin_amdgcn_sched_barrier(0);
@@ -571,6 +613,8 @@ int gmm_launch_persistent_probe(int parts_off, const f16* x, const f16* w, const
     AOPS_PROBE_CASE(kProbeNoXCopies | kProbeNoWCopies | kProbeNoFragments)  // 14: MFMAs only
     AOPS_PROBE_CASE(kProbeNoMfma)                                           // 1: copies and LDS fragment reads, no MFMAs
     AOPS_PROBE_CASE(kProbeNoFragments)                                      // 8: copies and MFMAs, no LDS fragment reads
+    AOPS_PROBE_CASE(kProbeWidePieces | kProbeNoMfma | kProbeNoFragments)                    // 25: as 9, weights in 256-byte pieces
+    AOPS_PROBE_CASE(kProbeWidePieces | kProbeNoMfma | kProbeNoFragments | kProbeNoXCopies)  // 27: as 11, weights in 256-byte pieces
 #undef AOPS_PROBE_CASE
     default:
       return AOPS_ERR_INVALID_ARGUMENT;

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ascend910a_extras operator set on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|norm|cache|rope|mlp|moe|moe_gate_up|moe_down|pa_more|dense|gmm_probe|scaled,...] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--ops all|norm|cache|rope|mlp|moe|moe_gate_up|moe_down|pa_more|dense|gmm_probe|gmm_probe_gate_up|gmm_probe_down|gmm_probe_dense|scaled,...] [--no-cpu]
 
 A "step" is one paged_attention decode call over the batch of BASELINE.json configs[4]
 (64 sequences, 32 query / 8 kv heads, head_dim 128, contexts ~U[512, 4096], block 128): the
@@ -848,7 +848,7 @@ def bench_dense(L, R, dev):
     return e
 
 
-def bench_gmm_probe(L, R, dev):
+def bench_gmm_probe(L, R, dev, only=None):
     """Where the time of the MoE GEMMs goes, from kernels in the library alone: the persistent grouped-matmul kernel
     on configs[3] with parts of its k loop switched off (aops_grouped_matmul_probe_f16), and a pure read stream
     with the access pattern of its weight copies next to a linear stream of the same bytes
@@ -862,6 +862,8 @@ def bench_gmm_probe(L, R, dev):
     out = []
     gl_moe, rows_moe = gl, rows
     for which, K, N in (("gate_up", hidden, 2 * inter), ("down", inter, hidden), ("dense", 8192, 8192)):
+        if only and which != only:   # one shape alone, so that a counter pass has one shape per kernel name
+            continue
         g = torch.Generator(device=dev).manual_seed(1)
         moe = which != "dense"   # the dense product: one group of 8192 rows (320-row tiles here, 256-row tiles in the "dense" line)
         E, rows = (128, rows_moe) if moe else (1, 8192)
@@ -886,7 +888,9 @@ def bench_gmm_probe(L, R, dev):
 
         for parts_off, what in ((0, "whole kernel"), (9, "operand copies and barriers only"), (11, "weight copies only"),
                                 (13, "activation copies only"), (6, "MFMAs and LDS fragment reads only"), (14, "MFMAs only"),
-                                (1, "copies and LDS fragment reads, no MFMAs"), (8, "copies and MFMAs, no LDS fragment reads")):
+                                (1, "copies and LDS fragment reads, no MFMAs"), (8, "copies and MFMAs, no LDS fragment reads"),
+                                (25, "operand copies and barriers only, weights in 256-byte pieces from half the rows per tile"),
+                                (27, "weight copies only, in 256-byte pieces from half the rows per tile")):
             med, mn = timed(parts_off)
             label = f"probe 4: MoE {which}" if moe else "probe dense 8192^3 (320-row tiles)"
             e = entry("grouped_matmul_probe", f"{label}, {what}", f"x [{rows},{K}] @ w [{E},{K},{N}] f16",
@@ -919,7 +923,9 @@ def bench_gmm_probe(L, R, dev):
         out.append(entry("grouped_matmul_ldw", f"probe 4: MoE {which}, weight rows padded to {2 * ldw} bytes (extension)",
                          f"x [{rows},{K}] @ w [{E},{K},{N}] f16, row stride {ldw}", "mfma", alg, flops, med, mn, None, None, 1,
                          "same kernel and same bits as the whole-kernel line; the caller pads the static weights once"))
-        for parts_off, what in ((9, "operand copies and barriers only"), (11, "weight copies only")):
+        for parts_off, what in ((9, "operand copies and barriers only"), (11, "weight copies only"),
+                                (25, "operand copies and barriers only, weights in 256-byte pieces"),
+                                (27, "weight copies only, in 256-byte pieces")):
             med, mn = timed(parts_off, wps, ldw)
             e = entry("grouped_matmul_probe", f"probe 4: MoE {which}, weight rows padded to {2 * ldw} bytes, {what}",
                       f"x [{rows},{K}] @ w [{E},{K},{N}] f16, row stride {ldw}", "mfma", alg, flops, med, mn, None, None, 1,
@@ -1043,6 +1049,9 @@ def main():
                         ("moe_gate_up_padded", lambda: bench_moe_one(L, ops, R, dev, "gate_up_padded")),
                         ("dense", lambda: bench_dense(L, R, dev)),
                         ("gmm_probe", lambda: bench_gmm_probe(L, R, dev)),
+                        ("gmm_probe_gate_up", lambda: bench_gmm_probe(L, R, dev, "gate_up")),
+                        ("gmm_probe_down", lambda: bench_gmm_probe(L, R, dev, "down")),
+                        ("gmm_probe_dense", lambda: bench_gmm_probe(L, R, dev, "dense")),
                         ("pa_more", lambda: bench_pa_more(L, R, dev, cpu))):
             if tag in want:
                 run(tag, fn)

@@ -359,8 +359,9 @@ int aops_probe_read_stream(const void* buf, int64_t rows, int64_t row_bytes, int
  * aops_grouped_matmul_ldw_f16 takes them).  parts_off: 9 = operand
  * copies and barriers only (no MFMAs, no LDS fragment reads), 11 = weight copies only, 13 = activation
  * copies only, 6 = MFMAs and fragment reads only (no copies), 14 = MFMAs only, 1 = everything but the MFMAs,
- * 8 = everything but the LDS fragment reads; anything else returns
- * AOPS_ERR_INVALID_ARGUMENT.  y is written with values that are wrong by construction.
+ * 8 = everything but the LDS fragment reads, 25 and 27 = 9 and 11 with the weight copies of a k tile taking
+ * 256 bytes of every row of half the tile's rows instead of 128 bytes of every row (the same requests in
+ * pieces twice as long); anything else returns AOPS_ERR_INVALID_ARGUMENT.  y is written with values that are wrong by construction.
  * No counterpart in the reference.
  */
 int aops_grouped_matmul_probe_f16(int parts_off, const void* x, const void* w, int64_t ldw,

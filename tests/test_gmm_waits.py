@@ -89,8 +89,8 @@ def test_scanner_flags_another_user_of_m0(assembly):
         ("__builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kBCopies));\n      fence();",
          "__builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(kBCopies + 1));\n      fence();", "expected s_waitcnt vmcnt"),
         # one weight copy fewer per tile than the waits assume
-        ("for (int i = 0; i < kBCopies; ++i) dma16(b_base + ko, b_offset(i), db + i * kWaves * 1024);",
-         "for (int i = 0; i < kBCopies - 1; ++i) dma16(b_base + ko, b_offset(i), db + i * kWaves * 1024);",
+        ("for (int i = 0; i < kBCopies; ++i)\n          if (kSlotsB > 0 && i * kSlotsB / kBCopies == slot) copy_w_one(kw, STAGE, i);",
+         "for (int i = 0; i < kBCopies - 1; ++i)\n          if (kSlotsB > 0 && i * kSlotsB / kBCopies == slot) copy_w_one(kw, STAGE, i);",
          "copies since"),
     ],
 )

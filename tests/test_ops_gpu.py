@@ -380,7 +380,7 @@ def test_measurement_aids_run_and_leave_their_surroundings_alone(dev):
     x, w, gl = _gmm_case(rows, K, N, E, seed=2, counts=[300, 0, 1, 330, 69])
     xd, wd, gd = x.to(dev), w.transpose(1, 2).contiguous().to(dev), gl.to(dev)
     y = torch.full((rows + 2, N), 7.0, dtype=H, device=dev)        # one guard row on either side
-    for parts_off in (9, 11, 13, 6, 14, 1, 8):
+    for parts_off in (9, 11, 13, 6, 14, 1, 8, 25, 27):
         assert lib.aops_grouped_matmul_probe_f16(parts_off, xd.data_ptr(), wd.data_ptr(), K, gd.data_ptr(),
                                                  y[1:].data_ptr(), rows, K, E, N, cabi.stream(dev)) == 0
     torch.cuda.synchronize()
