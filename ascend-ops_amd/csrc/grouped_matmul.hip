@@ -200,7 +200,9 @@ extern "C" int aops_grouped_matmul_swiglu_gather_f16(const void* x, const int32_
     return AOPS_ERR_INVALID_ARGUMENT;
   if (rows == 0 || num_experts == 0) return AOPS_OK;
   if (!x || !row_idx || !w || !group_list || !y) return AOPS_ERR_INVALID_ARGUMENT;
-  const int choice = fused_tile_choice(rows, k, num_experts);
+  int choice = fused_tile_choice(rows, k, num_experts);
+  // the persistent kernel addresses the gathered rows with 32-bit byte offsets: x below 4 GiB
+  if (choice == 0 && x_rows * k * 2 > 0xffffffffLL) choice = 1;
   if (choice != 0)
     return gmm_launch_tiles_fused(choice == 2, static_cast<const f16*>(x), static_cast<const f16*>(w),
                                   group_list, static_cast<f16*>(y), rows, (int)k, (int)num_experts, (int)n,

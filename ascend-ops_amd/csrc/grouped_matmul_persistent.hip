@@ -50,15 +50,25 @@ __device__ __forceinline__ int lane_id_fresh() {
 // checks both in the assembly of every instantiation at build time (no GPU needed): (1) M0 is written and
 // read by these copy sequences alone, and no register is spilled; (2) between two barriers of the k loop lie
 // exactly the copies the source issues there, and each barrier is directly preceded by its counted wait.
+// Per-lane byte offset of a copy: lane_base + uniform_add, clamped to cap.  Volatile asm, so that the nine
+// offsets of a tile's copies are computed where the copies are issued (two instructions each) instead of
+// being kept in registers across the k loop, where the accumulators fill the register file.
+__device__ __forceinline__ uint32_t copy_offset(uint32_t lane_base, uint32_t uniform_add, uint32_t cap) {
+  uint32_t r;
+  asm volatile("v_add_u32 %0, %1, %2\n\tv_min_u32 %0, %0, %3" : "=&v"(r) : "s"(uniform_add), "v"(lane_base), "v"(cap));
+  return r;
+}
+__device__ __forceinline__ uint32_t copy_offset(uint32_t lane_base, uint32_t uniform_add) {
+  uint32_t r;
+  asm volatile("v_add_u32 %0, %1, %2" : "=v"(r) : "s"(uniform_add), "v"(lane_base));
+  return r;
+}
+
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void dma16(const void* base, uint32_t lane_offset, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :: "s"(lds_addr), "v"(lane_offset), "s"(base) : "m0", "memory");
-}
-__device__ __forceinline__ void dma16(const void* lane_address, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-               :: "s"(lds_addr), "v"(lane_address) : "m0", "memory");
 }
 #pragma clang diagnostic pop
 
@@ -78,14 +88,15 @@ template <int MB, int NB, int WN, bool SWIGLU, bool GATHER, int PROBE = 0>
 __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kernel(
     const f16* __restrict__ x, const f16* __restrict__ w, const int64_t* __restrict__ group_list,
     f16* __restrict__ y, int64_t rows, int k, int num_experts, int n,
-    const int32_t* __restrict__ row_idx, int idx_div, uint32_t x_rows, int ldw) {
+    const int32_t* __restrict__ row_idx, uint32_t idx_magic, int idx_shift, uint32_t x_rows, int ldw) {
   constexpr int kWaves = 2 * WN;
   constexpr int BM = 64 * MB;
   constexpr int BN = 32 * NB * WN;
-  constexpr int kSteps = kBK / 16;
+  constexpr int kKSteps = kBK / 32;  // k steps of a tile: one v_mfma_f32_16x16x32_f16 deep each
   constexpr int kACopies = BM / 8 / kWaves;
   constexpr int kBCopies = BN / 8 / kWaves;
   static_assert(BM % (8 * kWaves) == 0 && BN % (8 * kWaves) == 0, "tile rows per copy");
+  static_assert(kKSteps == 2, "the k loop keeps the weight fragments of two k steps");
   static_assert(!SWIGLU || (NB == 2 && kWaves == 8), "gate/up pairing assumes 64-row copies, two column blocks");
   constexpr int BNO = SWIGLU ? BN / 2 : BN;  // output columns per work item
   const int n_out = SWIGLU ? n / 2 : n;      // output row length
@@ -190,9 +201,12 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
 #pragma unroll
       for (int i = 0; i < kACopies; ++i) {
         const int r = min(8 * kWaves * i + lane_row, x_left - 1);
-        uint32_t src = (uint32_t)row_idx[it.row_begin + r] / (uint32_t)idx_div;
+        // row_idx / idx_div as a multiplication (exact for indices below 2^31; the launcher derives the
+        // constants): a division by a run-time value costs a dozen registers that the k loop does not have
+        const uint32_t flat = (uint32_t)row_idx[it.row_begin + r];
+        uint32_t src = idx_magic ? (__umulhi(flat, idx_magic) >> idx_shift) : flat;
         src = src < x_rows ? src : x_rows - 1;  // an index outside x reads its last row instead of faulting
-        a_src[i] = src * (uint32_t)k + lane_c * 8;  // in elements: up to 2^32 of them
+        a_src[i] = (src * (uint32_t)k + lane_c * 8) * 2u;  // in bytes (the launcher refuses x of 4 GiB or more)
       }
     } else {
       a_base = x + (int64_t)it.row_begin * k;
@@ -202,9 +216,9 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   auto b_offset = [&](int i) -> uint32_t {
     if constexpr (SWIGLU) {
       const uint32_t blk = (uint32_t)i < b_last ? (uint32_t)i : 0u;  // blocks past n: repeat block 0
-      return off0_glu + blk * 64u * (uint32_t)ldw;
+      return copy_offset(off0_glu, blk * 64u * (uint32_t)ldw);
     } else {
-      return min(off0_w + i * copy_stride_w, b_last);
+      return copy_offset(off0_w, i * copy_stride_w, b_last);
     }
   };
   const uint32_t lds_sa = (uint32_t)(uintptr_t)AOPS_LDS_PTR(sa);  // LDS byte addresses of the stages
@@ -214,12 +228,12 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     if constexpr (PROBE & kProbeNoXCopies) return;
     const int ko = kt * kBK;
     const uint32_t da = lds_sa + (uint32_t)(stage * BM * kBK + wave * 512) * 2u;
-    if constexpr (GATHER) {  // offsets of up to 2^32 elements: 64-bit address per lane
-      dma16(a_base + ko + a_src[i], da + i * kWaves * 1024);
+    if constexpr (GATHER) {
+      dma16(a_base + ko, a_src[i], da + i * kWaves * 1024);
     } else {
       // uniform base + 32-bit byte offset per lane: the copy takes them as they are (scalar base,
       // vector offset), no vector instructions spent on a 64-bit address
-      dma16(a_base + ko, min(off0 + i * copy_stride, a_last), da + i * kWaves * 1024);
+      dma16(a_base + ko, copy_offset(off0, i * copy_stride, a_last), da + i * kWaves * 1024);
     }
   };
   auto copy_x = [&](int kt, int stage) {
@@ -244,19 +258,24 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     for (int i = 0; i < kBCopies; ++i) copy_w_one(kt, stage, i);
   };
 
-  const int fm = lane & 31;
-  const int fq = lane >> 5;
-  // Fragment addresses: lds_off(fm, 2*st + fq) == lds_off(fm, fq) ^ (st << 4) (the k step only
-  // flips two chunk bits), so one LDS byte address per operand and stage serves every k step: the
-  // step's XOR is one vector instruction, row block and column block are immediate offsets of the
-  // reads.  (Both regions start on 128-byte boundaries, so the XOR of bits 5-6 stays inside a row.)
+  // The MFMAs are v_mfma_f32_16x16x32_f16 (with operands that change from one instruction to the next the
+  // matrix cores run at the clock the power limit leaves them, and this shape sustains about a fifth more
+  // there than 32x32x16 does).  A fragment is 16 rows x 32 k: lane l holds row l & 15, k chunk l >> 4 (8 halfs).
+  const int fm = lane & 15;
+  const int fq = lane >> 4;
+  // Fragment addresses: lds_off(fm, 4*st + fq) == lds_off(fm, fq) ^ (st << 5) (the k step only flips the
+  // top chunk bit), so one LDS byte address per operand and stage serves both k steps: the step's XOR is one
+  // vector instruction, row block and column block are immediate offsets of the reads.  (Both regions start
+  // on 128-byte boundaries, so the XOR of bit 6 stays inside a row.)
   typedef const __attribute__((address_space(3))) f16x8* LdsFrag;
   const uint32_t fa_byte0 = lds_sa + (uint32_t)(lds_off(fm, fq) + wm * 32 * kBK) * 2u;
   const uint32_t fb_byte0 = lds_sb + (uint32_t)(lds_off(fm, fq) + wn * 32 * NB * kBK) * 2u;
   const uint32_t fa_byte[2] = {fa_byte0, fa_byte0 + BM * kBK * 2u};
   const uint32_t fb_byte[2] = {fb_byte0, fb_byte0 + BN * kBK * 2u};
 
-  f32x16 acc[MB][NB];
+  constexpr int JB = 2 * NB;  // 16-column blocks of a wave
+  // acc[b][j]: rows 32*(wm + 2*(b/2)) + 16*(b%2) .. +15 of the tile, columns 16*j .. +15 of the wave
+  f32x4 acc[2 * MB][JB];
   GmmWork nxt;
 
   // The k loop.  Per k tile t (stage t & 1) a wave reads its weight fragments of all four k steps into
@@ -276,9 +295,10 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
   // tile t+2 when the next ones arrive, instead of draining to empty at every barrier.
   auto k_loop = [&](auto live_c) {
     constexpr int LIVE = decltype(live_c)::value;
-    constexpr int NF = kSteps * LIVE;  // activation fragments (pairs of MFMAs) of a k tile
-    constexpr int kFa = 4;             // activation fragments in flight
-    f16x8 fa[LIVE > 0 ? kFa : 1], fb[kSteps][NB];
+    constexpr int NBLK = 2 * LIVE;         // 16-row blocks of this wave that hold rows of the group
+    constexpr int NF = kKSteps * NBLK;     // activation fragments of a k tile, JB MFMAs each
+    constexpr int kFa = 4;                 // activation fragments in flight
+    f16x8 fa[LIVE > 0 ? kFa : 1], fb[kKSteps][JB];
     if constexpr (PROBE & kProbeNoFragments) {  // operands the compiler cannot fold: the MFMAs stay
       const f16x8 one = {1, 1, 1, 1, 1, 1, 1, 1};
       for (auto& f : fa) {
@@ -293,32 +313,35 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     }
     // The XORs are volatile asm: written as expressions they would be hoisted out of the k loop, one
     // address register per (operand, stage, step), and push the accumulators into scratch.
-    auto read_fb = [&](auto st_c, auto stage_c) {
+    auto read_fb = [&](auto st_c, auto stage_c) {  // the weight fragments of k step ST
       constexpr int ST = decltype(st_c)::value;
       constexpr int STAGE = decltype(stage_c)::value;
       if constexpr (PROBE & kProbeNoFragments) return;
       uint32_t pb = fb_byte[STAGE];
-      if constexpr (ST > 0) asm volatile("v_xor_b32 %0, %1, %2" : "=v"(pb) : "n"(ST << 5), "v"(fb_byte[STAGE]));
+      if constexpr (ST > 0) asm volatile("v_xor_b32 %0, %1, %2" : "=v"(pb) : "n"(ST << 6), "v"(fb_byte[STAGE]));
 #pragma unroll
-      for (int j = 0; j < NB; ++j) fb[ST][j] = *reinterpret_cast<LdsFrag>(pb + j * 32 * kBK * 2);
+      for (int j = 0; j < JB; ++j) fb[ST][j] = *reinterpret_cast<LdsFrag>(pb + j * 16 * kBK * 2);
     };
-    auto read_fa = [&](auto n_c, auto stage_c) {  // fragment n = (row block n / kSteps, k step n % kSteps)
+    // fragment n = (k step n / NBLK, 16-row block n % NBLK): k step by k step, so that the last kTail fragments
+    // of a tile all belong to its last k step and the registers of the first are free for the next tile's
+    // weights while they run
+    auto read_fa = [&](auto n_c, auto stage_c) {
       constexpr int N = decltype(n_c)::value;
       constexpr int STAGE = decltype(stage_c)::value;
       if constexpr (N >= 0 && N < NF && !(PROBE & kProbeNoFragments)) {
-        constexpr int ST = N % kSteps;
+        constexpr int ST = N % kKSteps;
+        constexpr int B = N / kKSteps;
         uint32_t pa = fa_byte[STAGE];
-        if constexpr (ST > 0) asm volatile("v_xor_b32 %0, %1, %2" : "=v"(pa) : "n"(ST << 5), "v"(fa_byte[STAGE]));
-        fa[N % kFa] = *reinterpret_cast<LdsFrag>(pa + (N / kSteps) * 64 * kBK * 2);
+        if constexpr (ST > 0) asm volatile("v_xor_b32 %0, %1, %2" : "=v"(pa) : "n"(ST << 6), "v"(fa_byte[STAGE]));
+        fa[N % kFa] = *reinterpret_cast<LdsFrag>(pa + ((B / 2) * 64 + (B % 2) * 16) * kBK * 2);
       }
     };
     auto mma = [&](auto n_c) {
       constexpr int N = decltype(n_c)::value;
       if constexpr (N >= 0 && N < NF && !(PROBE & kProbeNoMfma)) {
 #pragma unroll
-        for (int j = 0; j < NB; ++j)
-          acc[N / kSteps][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[N % kSteps][j], fa[N % kFa],
-                                                                      acc[N / kSteps][j], 0, 0, 0);
+        for (int j = 0; j < JB; ++j)
+          acc[N / kKSteps][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[N % kKSteps][j], fa[N % kFa], acc[N / kKSteps][j], 0, 0, 0);
       }
     };
     auto fence = [] {
@@ -337,9 +360,13 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
         self(self, std::integral_constant<int, N + 1>{}, end_c, stage_c, hook);
       }
     };
-    // The last kTail pairs of a tile run at the start of the next one, between its first fragment reads,
-    // so that the matrix cores have work while those reads are on their way.
-    constexpr int kTail = kSteps;  // = kFa: the tail holds the whole fragment ring and every weight step
+    // The MFMAs of the last kTail fragments of a tile run at the start of the next one, between its first
+    // fragment reads, so that the matrix cores have work while those reads are on their way.  The tail is
+    // the whole fragment ring; it needs the weight fragments of the tile's last k step (and, with two blocks
+    // per wave, for its first half those of the first), which the next tile's reads may only replace after
+    // the tail MFMAs that use them.
+    constexpr int kTail = kFa;
+    constexpr int kFbStart0 = NBLK >= kTail ? 0 : kTail / 2 - 1;  // start() call that reads the weights of k step 0
     // barrier B comes after this many pairs of the tile: the burst of reads at its start has returned by
     // then, so the wait in front of the barrier costs nothing
     constexpr int kPairsBeforeB = NF - kTail < 6 ? NF - kTail : 6;
@@ -372,7 +399,8 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
           x_copies_of_slot(Q);
           read_fa(q_c, stage_c);
           __builtin_amdgcn_sched_barrier(0);  // the counted wait in front of barrier B relies on this order
-          read_fb(q_c, stage_c);
+          if constexpr (Q == 2) read_fb(std::integral_constant<int, 0>{}, stage_c);
+          if constexpr (Q == kTail - 1) read_fb(std::integral_constant<int, 1>{}, stage_c);
           __builtin_amdgcn_sched_barrier(0);
         };
         start(std::integral_constant<int, 0>{});
@@ -436,11 +464,12 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     const int live_blocks = (tile_rows + 31) / 32;
     const int live = (live_blocks - wm + 1) / 2;
 #pragma unroll
-    for (int i = 0; i < MB; ++i)
+    for (int b = 0; b < 2 * MB; ++b)
 #pragma unroll
-      for (int j = 0; j < NB; ++j)
+      for (int j = 0; j < JB; ++j) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        for (int r = 0; r < 4; ++r) acc[b][j][r] = 0.f;
+      }
 
     if (live >= MB) {
       k_loop(std::integral_constant<int, MB>{});
@@ -454,29 +483,31 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
       k_loop(std::integral_constant<int, 0>{});
     }
 
-    // Epilogue of `cur`.  acc[i][j][4g+e]: output row 32*(wm+2i) + fm, output column
-    // wn*32*NB + 32j + 8g + 4fq + e: a lane holds one output row and, of the wave's columns, 8-byte
-    // pieces that alternate with those of its partner lane (fq).  Stored from there, every store
-    // instruction would scatter 32-byte pieces over 32 rows, and the count of write requests, not their
+    // Epilogue of `cur`.  acc[b][j][e]: output row 32*(wm + 2*(b/2)) + 16*(b%2) + fm, output column
+    // wn*32*NB + 16j + 4fq + e: a lane holds one output row of a 16-row block and, of the wave's columns,
+    // 8-byte pieces that alternate with those of three other lanes.  Stored from there, every store
+    // instruction would scatter 8-byte pieces over 16 rows, and the count of write requests, not their
     // bytes, is what the memory pipeline of a CU charges for.  So the rows go through a 1 KiB LDS scratch
     // of the wave's own, a few at a time: the lanes of those rows write their pieces (16-byte slots
-    // XOR-swizzled by the row: no bank conflicts either way), then all 64 lanes read 16 bytes each in row
-    // order and store whole row segments - eight 128-byte lines per instruction (SWIGLU: sixteen 64-byte
-    // halves).  The operand stages stay untouched: the next item's first tiles are landing in them.
+    // XOR-swizzled by the row: no bank conflicts beyond the two cycles that 256 bytes take), then all 64
+    // lanes read 16 bytes each in row order and store whole row segments - eight 128-byte lines per
+    // instruction (SWIGLU: sixteen 64-byte halves).  The operand stages stay untouched: the next item's
+    // first tiles are landing in them.
     {
       f16* scr = sepi + wave * kEpiScratchHalfs;
       constexpr int kSegHalfs = SWIGLU ? 32 : 32 * NB;       // output columns of the wave
       constexpr int kRowsPerUnit = kEpiScratchHalfs / kSegHalfs;  // 8 rows of 128 bytes, or 16 of 64
       constexpr int kSlots = kSegHalfs / 8;                  // 16-byte slots per row segment
-      constexpr int kUnits = 32 / kRowsPerUnit;
+      constexpr int kUnits = 16 / kRowsPerUnit;              // per 16-row block
+      constexpr int kOutBlocks = kSegHalfs / 16;             // 16-column blocks of the wave's output
       static_assert(kSegHalfs == 128 || kSegHalfs == 64 || kSegHalfs == 32, "row segment of 256, 128 or 64 bytes");
-      static_assert(kRowsPerUnit <= 32 && 32 % kRowsPerUnit == 0 && kRowsPerUnit * kSlots == kWave, "one 16-byte slot per lane");
+      static_assert(kRowsPerUnit <= 16 && 16 % kRowsPerUnit == 0 && kRowsPerUnit * kSlots == kWave, "one 16-byte slot per lane");
       const int col_w = SWIGLU ? cur.n_tile * BNO + wn * 32 : cur.n_tile * BN + wn * 32 * NB;
       // the lane-derived offsets are the same for every item; taken from a fresh lane id they are not
       // hoisted out of the item loop (and spilled)
       const int lane_e = lane_id_fresh();
-      const int fm_e = lane_e & 31;
-      const int fq_e = lane_e >> 5;
+      const int fm_e = lane_e & 15;
+      const int fq_e = lane_e >> 4;
       const int unit_of_lane = fm_e / kRowsPerUnit;
       const int r_w = fm_e % kRowsPerUnit;                    // this lane's row inside its unit
       const int r_r = lane_e / kSlots;                        // the row this lane reads back and stores
@@ -484,28 +515,31 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
       // slot swizzle of row r: rows whose segments start in the same bank get different slot orders
       auto swz = [](int r) { return kSlots == 16 ? (r & 3) : kSlots == 8 ? (r & 7) : ((r ^ (r >> 2)) & 3); };
       const f16* rd = scr + r_r * kSegHalfs + ((q_r ^ swz(r_r)) * 8);
+      // this lane's pieces of a row: columns 16*jj + 4*fq .. +3, i.e. slot 2*jj + fq/2, its half fq%2
+      f16* wr = scr + r_w * kSegHalfs + 4 * (fq_e & 1);
+      const int q_w = (fq_e >> 1) ^ swz(r_w);                 // (2*jj + fq/2) ^ swz == (2*jj) ^ q_w: swz < kSlots
 #pragma unroll
-      for (int i = 0; i < MB; ++i) {
-        if (i < live && col_w < n_out) {  // wave uniform
+      for (int b = 0; b < 2 * MB; ++b) {
+        if (b / 2 < live && col_w < n_out) {  // wave uniform
           // (the conversion sits inside the branch of the lane's unit: no registers are held for the pieces)
 #pragma unroll
           for (int u = 0; u < kUnits; ++u) {
             if (unit_of_lane == u) {
 #pragma unroll
-              for (int q = 0; q < kSlots; ++q) {
-                f16x4 piece;  // slot q of this lane's row, its fq half
+              for (int jj = 0; jj < kOutBlocks; ++jj) {
+                f16x4 piece;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                   if constexpr (SWIGLU) {
-                    const float gt = acc[i][0][4 * q + e];
-                    const float up = acc[i][1][4 * q + e];
+                    const float gt = acc[b][jj][e];
+                    const float up = acc[b][jj + JB / 2][e];
                     const float ex = __builtin_amdgcn_exp2f(-1.4426950408889634f * gt);
                     piece[e] = (f16)(gt * up * __builtin_amdgcn_rcpf(1.0f + ex));
                   } else {
-                    piece[e] = (f16)acc[i][q / 4][4 * (q % 4) + e];
+                    piece[e] = (f16)acc[b][jj][e];
                   }
                 }
-                *reinterpret_cast<f16x4*>(scr + r_w * kSegHalfs + ((q ^ swz(r_w)) * 8) + 4 * fq_e) = piece;
+                *reinterpret_cast<f16x4*>(wr + (((2 * jj) ^ q_w) * 8)) = piece;
               }
             }
             // LDS serves a wave's accesses in order: the read sees the writes above, and the next unit's
@@ -513,7 +547,7 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
             asm volatile("" ::: "memory");
             const f16x8 v = *reinterpret_cast<const f16x8*>(rd);
             asm volatile("" ::: "memory");
-            const int m = 32 * wm + 64 * i + u * kRowsPerUnit + r_r;
+            const int m = 32 * wm + 64 * (b / 2) + 16 * (b % 2) + u * kRowsPerUnit + r_r;
             if (m < tile_rows)
               st128_stream(y + (int64_t)(cur.row_begin + m) * n_out + col_w + q_r * 8, v);
           }
@@ -551,8 +585,18 @@ static int gmm_persistent_launch(const f16* x, const f16* w, const int64_t* grou
   static std::atomic<uint64_t> lds_allowed{0};  // per device
   if (const hipError_t le = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLds, lds_allowed); le != hipSuccess)
     return record_launch_status(le);
+  // idx_div >= 2: q = (flat * magic) >> (32 + shift) with magic = ceil(2^(31 + l) / idx_div), l = ceil(log2 idx_div),
+  // shift = l - 1; exact for flat < 2^31.  idx_div == 1: magic 0 = no division.
+  uint32_t idx_magic = 0;
+  int idx_shift = 0;
+  if (idx_div >= 2) {
+    int l = 0;
+    while ((1ll << l) < idx_div) ++l;
+    idx_magic = (uint32_t)(((1ull << (31 + l)) + (uint64_t)idx_div - 1) / (uint64_t)idx_div);
+    idx_shift = l - 1;
+  }
   kernel<<<(unsigned)grid, 2 * WN * kWave, kLds, stream>>>(x, w, group_list, y, rows, k, num_experts,
-                                                          n, row_idx, idx_div, (uint32_t)x_rows, ldw);
+                                                          n, row_idx, idx_magic, idx_shift, (uint32_t)x_rows, ldw);
   return record_launch_status(hipGetLastError());
 }
 
@@ -582,6 +626,7 @@ int gmm_launch_persistent(bool swiglu, const f16* x, const f16* w, const int64_t
   const int64_t n_out_tiles = swiglu ? (n / 2 + 127) / 128 : (n + 255) / 256;
   const bool small = gmm_prefer_256_rows(rows, num_experts, n_out_tiles, device_cu_count());
   if (row_idx) {  // only the fused gate_up form gathers
+    if (x_rows * k * 2 > 0xffffffffLL) return AOPS_ERR_INVALID_ARGUMENT;  // 32-bit byte offsets into x
     if (small)
       return gmm_persistent_launch<4, 2, 4, true, true>(x, w, group_list, y, rows, k, num_experts, n, stream,
                                                         row_idx, idx_div, x_rows, ldw);
