@@ -260,9 +260,13 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
 
   // The MFMAs are v_mfma_f32_16x16x32_f16 (with operands that change from one instruction to the next the
   // matrix cores run at the clock the power limit leaves them, and this shape sustains about a fifth more
-  // there than 32x32x16 does).  A fragment is 16 rows x 32 k: lane l holds row l & 15, k chunk l >> 4 (8 halfs).
+  // there than 32x32x16 does).  A fragment is 16 rows x 32 k: lane l holds row l & 15 and the l >> 4'th group of 8
+  // k values.  Which 16-byte chunk of the tile's row a group is taken from is free as long as both operands
+  // take the same one (the sum over k does not care about the order): lanes l and l + 32 are served by LDS in
+  // the same cycle, and with chunks 0, 2, 1, 3 for l >> 4 = 0 .. 3 their chunks differ in the lowest bit, which
+  // the row swizzle turns into different bank halves (chunks l >> 4 as they come: every read a two-way conflict).
   const int fm = lane & 15;
-  const int fq = lane >> 4;
+  const int fq = ((lane >> 4) & 1) * 2 + (lane >> 5);
   // Fragment addresses: lds_off(fm, 4*st + fq) == lds_off(fm, fq) ^ (st << 5) (the k step only flips the
   // top chunk bit), so one LDS byte address per operand and stage serves both k steps: the step's XOR is one
   // vector instruction, row block and column block are immediate offsets of the reads.  (Both regions start

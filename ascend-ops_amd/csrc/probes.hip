@@ -8,6 +8,9 @@
 //    reads its 128 x seg_bytes block linearly.  No arithmetic beyond a sum that keeps the loads alive.  The bytes
 //    go into registers or, like the operand copies of the persistent grouped-matmul kernel, straight into LDS.
 //  * aops_grouped_matmul_probe_f16: the persistent grouped-matmul kernel with parts of its k loop switched off.
+//  * aops_probe_mfma_rate: fp16 MFMAs of one shape on operands held in registers and nothing else - the rate the
+//    matrix cores sustain for a given operand content (all-zero operands: the peak; operands that change from one
+//    instruction to the next: what the power limit leaves).
 #include "gmm_common.h"
 
 namespace aops {
@@ -54,7 +57,74 @@ __global__ __launch_bounds__(256) void probe_read_stream_kernel(const char* __re
   if (acc[0] + acc[1] + acc[2] + acc[3] == 12345.678f) sink[0] = acc[0];
 }
 
+// Every wave issues `iters` rounds of MFMAs of 8 x 16384 multiply-adds' worth (8 of 32x32x16 or 16 of 16x16x32) on
+// eight A and eight B fragments read once from `operands`; every instruction takes another pair of them than the
+// one before, and the accumulators (128 registers either way) are independent.
+template <int SHAPE>
+__global__ __launch_bounds__(512) void probe_mfma_rate_kernel(const f16x8* __restrict__ operands, float* __restrict__ sink,
+                                                              int iters) {
+  const int lane = threadIdx.x & (kWave - 1);
+  f16x8 a[8], b[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = operands[i * kWave + lane];
+    b[i] = operands[(i + 8) * kWave + lane];
+  }
+  float total = 0.f;
+  if constexpr (SHAPE == 32) {
+    f32x16 acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+    for (int it = 0; it < iters; it += 8) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[(i + 3 * j) & 7], b[(i + j) & 7], acc[i], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) total += acc[i][r];
+  } else {
+    f32x4 acc[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[i][r] = 0.f;
+    for (int it = 0; it < iters; it += 8) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          acc[i + 16 * (j & 1)] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[(i + 3 * j) & 7], b[(i + j) & 7],
+                                                                         acc[i + 16 * (j & 1)], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 32; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) total += acc[i][r];
+  }
+  // never true for finite operands: the store only keeps the MFMAs alive
+  if (total == 12345.678f) sink[0] = total;
+}
+
 }  // namespace aops
+
+extern "C" int aops_probe_mfma_rate(int shape, const void* operands, int64_t iters, void* sink, void* stream) {
+  using namespace aops;
+  if ((shape != 16 && shape != 32) || !operands || !sink || iters <= 0 || iters % 8 != 0 || iters > (1 << 20))
+    return AOPS_ERR_INVALID_ARGUMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const unsigned grid = (unsigned)device_cu_count();
+  if (shape == 32)
+    probe_mfma_rate_kernel<32><<<grid, 512, 0, s>>>(static_cast<const f16x8*>(operands), static_cast<float*>(sink), (int)iters);
+  else
+    probe_mfma_rate_kernel<16><<<grid, 512, 0, s>>>(static_cast<const f16x8*>(operands), static_cast<float*>(sink), (int)iters);
+  return record_launch_status(hipGetLastError());
+}
 
 extern "C" int aops_probe_read_stream(const void* buf, int64_t rows, int64_t row_bytes, int64_t seg_bytes,
                                       int via_lds, void* sink, void* stream) {

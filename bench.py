@@ -898,10 +898,24 @@ def bench_gmm_probe(L, R, dev, only=None):
                       None if parts_off == 0 else "parts of the k loop switched off: results wrong by construction, time only")
             e["parts_off"] = parts_off
             out.append(e)
+        # the same launch on operands that are all zero: the matrix cores' multipliers do not switch, the chip
+        # stays inside its power limit at full clock, and what is left is the time of the operand copies
+        for i in range(sets):
+            xs[i].zero_()
+            ws[i].zero_()
+        med, mn = timed(0)
+        label = f"probe 4: MoE {which}" if moe else "probe dense 8192^3 (320-row tiles)"
+        out.append(entry("grouped_matmul_probe", f"{label}, whole kernel on all-zero operands",
+                         f"x [{rows},{K}] @ w [{E},{K},{N}] f16", "mfma", alg, flops, med, mn, None, None, 1,
+                         "the same launch as the whole-kernel line, correct results (zeros); the difference to that line "
+                         "is what the power limit costs with operands that change"))
         if not moe:
             del xs, ws, ys
             torch.cuda.empty_cache()
             continue
+        g = torch.Generator(device=dev).manual_seed(1)   # back to the operands of the lines above
+        xs = [torch.randn(rows, K, generator=g, device=dev, dtype=torch.float16) for _ in range(sets)]
+        ws = [torch.randn(E, N, K, generator=g, device=dev, dtype=torch.float16) * 0.02 for _ in range(sets)]
         # the same GEMM on weights whose rows are padded by one cache line (aops_grouped_matmul_ldw_f16): what the
         # power-of-two row stride of the reference's layout costs
         ldw = K + 64
@@ -956,6 +970,22 @@ def bench_gmm_probe(L, R, dev, only=None):
                              None, None, 1))
         del xs, ws, ys
         torch.cuda.empty_cache()
+    if only is None:
+        # what the matrix cores sustain by themselves: fp16 MFMAs of the two shapes on operands in registers
+        sink = torch.zeros(1, dtype=torch.float32, device=dev)
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        iters = 8192
+        flops = cus * 8 * iters * 8 * 32768
+        gen = torch.Generator(device=dev).manual_seed(3)
+        for data, operands in (("all-zero operands", torch.zeros(16 * 64 * 8, device=dev, dtype=torch.float16)),
+                               ("operands uniform in [-2, 2)", (torch.rand(16 * 64 * 8, generator=gen, device=dev) * 4 - 2).half())):
+            for shape, name in ((32, "v_mfma_f32_32x32x16_f16"), (16, "v_mfma_f32_16x16x32_f16")):
+                calls = [lambda: L.check(L.lib.aops_probe_mfma_rate(shape, operands.data_ptr(), iters, sink.data_ptr(), L.stream()))]
+                med, mn = time_graph(calls, min_launches=6, trials=3)
+                out.append(entry("mfma_rate_probe", f"probe: {name} alone, {data}", f"{cus} CUs x 8 waves x {iters} rounds",
+                                 "mfma", 16384 * cus * 8, flops, med, mn, None, None, 1,
+                                 "MFMAs on registers, nothing else: the rate the matrix cores sustain for this operand content"))
+
     return out
 
 

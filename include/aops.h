@@ -353,6 +353,17 @@ int aops_probe_read_stream(const void* buf, int64_t rows, int64_t row_bytes, int
                            void* sink, void* stream);
 
 /*
+ * Measurement aid: the rate at which the matrix cores execute fp16 MFMAs of one shape (shape 32:
+ * v_mfma_f32_32x32x16_f16, shape 16: v_mfma_f32_16x16x32_f16) on operands held in registers, with nothing else
+ * going on.  One workgroup of eight waves per CU; every wave reads sixteen fragments (16 KiB of fp16 at
+ * `operands`, device memory) once and then issues iters (a multiple of 8, at most 2^20) rounds of MFMAs worth
+ * 8 x 16384 multiply-adds each, so a launch does CUs x 8 x iters x 8 x 32768 flop.  With all-zero operands the
+ * result is the peak; with operands that differ from one instruction to the next it is what the power limit
+ * leaves.  sink: 4 bytes of device memory (never written for finite operands).  No counterpart in the reference.
+ */
+int aops_probe_mfma_rate(int shape, const void* operands, int64_t iters, void* sink, void* stream);
+
+/*
  * Measurement aid: the persistent 320 x 256 kernel of aops_grouped_matmul_f16 (k % 128 == 0, k >= 256)
  * with parts of its k loop switched off, to time what the rest costs by itself.  ldw = elements from one
  * weight row to the next (k: densely packed, as the operator takes them; more: padded rows, as

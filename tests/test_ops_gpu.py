@@ -404,6 +404,13 @@ def test_measurement_aids_run_and_leave_their_surroundings_alone(dev):
     assert lib.aops_probe_read_stream(buf.data_ptr(), 256, 1024, 96, 0, sink.data_ptr(), cabi.stream(dev)) == -1    # piece size
     assert lib.aops_probe_read_stream(buf.data_ptr(), 256, 640, 256, 0, sink.data_ptr(), cabi.stream(dev)) == -1    # not dividing
     assert lib.aops_probe_read_stream(buf.data_ptr(), 256, 1024, 128, 2, sink.data_ptr(), cabi.stream(dev)) == -1   # via_lds
+    operands = (torch.rand(16 * 64 * 8, device=dev) - 0.5).half()
+    for shape in (16, 32):
+        assert lib.aops_probe_mfma_rate(shape, operands.data_ptr(), 64, sink.data_ptr(), cabi.stream(dev)) == 0
+    torch.cuda.synchronize()
+    assert float(sink[0]) == 0.0
+    for shape, iters in ((8, 64), (16, 0), (16, 12), (32, (1 << 20) + 8)):
+        assert lib.aops_probe_mfma_rate(shape, operands.data_ptr(), iters, sink.data_ptr(), cabi.stream(dev)) == -1
 
 
 @pytest.mark.parametrize("seed", range(12))
