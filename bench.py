@@ -892,7 +892,8 @@ def bench_gmm_probe(L, R, dev, only=None):
                                 (25, "operand copies and barriers only, weights in 256-byte pieces from half the rows per tile"),
                                 (27, "weight copies only, in 256-byte pieces from half the rows per tile")):
             med, mn = timed(parts_off)
-            label = f"probe 4: MoE {which}" if moe else "probe dense 8192^3 (320-row tiles)"
+            # the whole kernel goes through the library's own choice of tile height (256 rows for the dense product)
+            label = f"probe 4: MoE {which}" if moe else f"probe dense 8192^3 ({256 if parts_off == 0 else 320}-row tiles)"
             e = entry("grouped_matmul_probe", f"{label}, {what}", f"x [{rows},{K}] @ w [{E},{K},{N}] f16",
                       "mfma", alg, flops, med, mn, None, None, 1,
                       None if parts_off == 0 else "parts of the k loop switched off: results wrong by construction, time only")
@@ -904,7 +905,7 @@ def bench_gmm_probe(L, R, dev, only=None):
             xs[i].zero_()
             ws[i].zero_()
         med, mn = timed(0)
-        label = f"probe 4: MoE {which}" if moe else "probe dense 8192^3 (320-row tiles)"
+        label = f"probe 4: MoE {which}" if moe else "probe dense 8192^3 (256-row tiles)"
         out.append(entry("grouped_matmul_probe", f"{label}, whole kernel on all-zero operands",
                          f"x [{rows},{K}] @ w [{E},{K},{N}] f16", "mfma", alg, flops, med, mn, None, None, 1,
                          "the same launch as the whole-kernel line, correct results (zeros); the difference to that line "
