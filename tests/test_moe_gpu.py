@@ -4,6 +4,7 @@ whole routed MLP are compared in fp32 within the grouped-matmul tolerance."""
 import pytest
 import torch
 
+import cabi
 import oracle.ops_ref as R
 
 pytestmark = pytest.mark.gpu
@@ -109,6 +110,32 @@ def test_gather_fused_gate_up_equals_gather_then_matmul(dev, tokens, topk, E, hi
     b = C.grouped_matmul_swiglu(moe.moe_gather(x, s, gl, topk), w1, gl)
     assert a.shape == (tokens * topk, inter)
     assert torch.equal(a[:end], b[:end])
+
+
+@pytest.mark.parametrize("x_bytes", [(1 << 32) - (1 << 20), (1 << 32) + (1 << 22)])
+def test_gather_fused_gate_up_reaches_rows_on_both_sides_of_4_gib(dev, x_bytes):
+    """The persistent kernel addresses the gathered rows with 32-bit byte offsets, so an activation matrix of 4 GiB or
+    more goes to the tile kernels instead: rows from the far end of x, just below and just above that size, against the
+    explicit gather followed by the matmul."""
+    import ascend910a_extras.ascend910a_extras_C as C
+    hidden, inter, E, per = 2048, 128, 4, 256
+    tokens = x_bytes // (2 * hidden)
+    g = torch.Generator().manual_seed(11)
+    x = torch.zeros(tokens, hidden, dtype=H, device=dev)
+    picked = torch.cat([torch.randint(0, tokens, (E * per - 64,), generator=g), torch.arange(tokens - 64, tokens)])
+    picked = picked[torch.randperm(E * per, generator=g)].to(torch.int32)
+    rows = torch.randn(E * per, hidden, generator=g).half()
+    x[picked.long().to(dev)] = rows.to(dev)      # duplicates in `picked`: the last write wins, both sides read x afterwards
+    w1 = (torch.randn(E, 2 * inter, hidden, generator=g) / hidden ** 0.5).half().to(dev)   # [E, N, K]: the C ABI's layout
+    gl = (torch.arange(1, E + 1, dtype=torch.int64) * per).to(dev)
+    s = picked.to(dev)
+    a = torch.empty(E * per, inter, dtype=H, device=dev)
+    # through the C ABI: the Python operator insists on one index per (token, choice), the boundary does not
+    assert cabi.lib().aops_grouped_matmul_swiglu_gather_f16(x.data_ptr(), s.data_ptr(), 1, tokens, w1.data_ptr(), gl.data_ptr(),
+                                                            a.data_ptr(), E * per, hidden, E, 2 * inter, cabi.stream(dev)) == 0
+    b = C.grouped_matmul_swiglu(x[s.long()], w1.transpose(1, 2), gl)
+    torch.testing.assert_close(a.float(), b.float(), rtol=2e-2, atol=2e-2)
+    assert float(a.float().abs().mean()) > 0.01
 
 
 @pytest.mark.parametrize("tokens,topk,E,hidden,inter", [(50, 2, 300, 384, 64), (64, 8, 128, 512, 256), (8, 8, 16, 256, 128),
