@@ -93,7 +93,11 @@ def test_moe_mlp_end_to_end(dev, tokens, topk, E, hidden, inter):
     torch.testing.assert_close(out.cpu().float(), ref, rtol=2e-2, atol=2e-2)
 
 
-@pytest.mark.parametrize("tokens,topk,E,hidden,inter", [(700, 4, 16, 256, 128), (4096, 8, 128, 512, 384), (50, 2, 300, 384, 64)])
+@pytest.mark.parametrize("tokens,topk,E,hidden,inter", [(700, 4, 16, 256, 128), (4096, 8, 128, 512, 384), (50, 2, 300, 384, 64),
+                                                         # top-k that is not a power of two (the persistent kernel divides the
+                                                         # flat index by it with a multiplication), enough rows per expert for it
+                                                         (600, 3, 8, 256, 128), (500, 7, 16, 384, 64), (900, 5, 20, 256, 64),
+                                                         (400, 6, 10, 512, 64), (300, 11, 12, 256, 64)])
 def test_gather_fused_gate_up_equals_gather_then_matmul(dev, tokens, topk, E, hidden, inter):
     """The grouped matmul that reads its rows through the routing order against the explicit gather followed by the
     same kernel without the index: bit for bit (same arithmetic, same order), invalid ids included."""
