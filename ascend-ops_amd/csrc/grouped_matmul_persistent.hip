@@ -19,8 +19,8 @@ namespace aops {
 // kernel writes y[r, c] = silu(h[r, c]) * h[r, d + c] (h = x @ W_e^T in fp32, never stored) as a
 // [rows, d] matrix.  A work item then covers 32*WN output columns; the weight stage holds, for wave
 // column wn, the 32 gate rows of its columns in row block 2*wn and the matching 32 up rows in row
-// block 2*wn + 1, so that a lane finds gate and up value of one output element in acc[i][0] and
-// acc[i][1].
+// block 2*wn + 1, so that a lane finds gate and up value of one output element in acc[b][j] and
+// acc[b][j + 2] (16-column blocks j = 0, 1 of the gate rows, 2, 3 of the up rows).
 //
 // GATHER = true reads the activation rows through an index: sorted row j comes from row
 // row_idx[j] / idx_div of x (the routing order of a mixture of experts: row_idx = the sorted flat
@@ -326,9 +326,8 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
 #pragma unroll
       for (int j = 0; j < JB; ++j) fb[ST][j] = *reinterpret_cast<LdsFrag>(pb + j * 16 * kBK * 2);
     };
-    // fragment n = (k step n / NBLK, 16-row block n % NBLK): k step by k step, so that the last kTail fragments
-    // of a tile all belong to its last k step and the registers of the first are free for the next tile's
-    // weights while they run
+    // fragment n = (16-row block n / 2, k step n % 2): row block by row block (taken k step by k step the
+    // compiler needs 40 registers more and spills)
     auto read_fa = [&](auto n_c, auto stage_c) {
       constexpr int N = decltype(n_c)::value;
       constexpr int STAGE = decltype(stage_c)::value;
@@ -352,9 +351,9 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
       asm volatile("" ::: "memory");
       __builtin_amdgcn_sched_barrier(0);
     };
-    // MFMA pairs N .. END-1 of the tile, each followed by the copies that hook(N) issues and by the read of the
-    // fragment that takes the pair's place
-    auto pairs = [&](auto self, auto n_c, auto end_c, auto stage_c, auto&& hook) {
+    // The MFMA groups of fragments N .. END-1 of the tile (JB MFMAs each, one per 16-column block of the wave), each
+    // followed by the copies that hook(N) issues and by the read of the fragment that takes this one's place
+    auto groups = [&](auto self, auto n_c, auto end_c, auto stage_c, auto&& hook) {
       constexpr int N = decltype(n_c)::value;
       if constexpr (N < decltype(end_c)::value) {
         mma(n_c);
@@ -366,22 +365,22 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
     };
     // The MFMAs of the last kTail fragments of a tile run at the start of the next one, between its first
     // fragment reads, so that the matrix cores have work while those reads are on their way.  The tail is
-    // the whole fragment ring; it needs the weight fragments of the tile's last k step (and, with two blocks
-    // per wave, for its first half those of the first), which the next tile's reads may only replace after
-    // the tail MFMAs that use them.
+    // the whole fragment ring: the last two row blocks at both k steps, so tail group q needs the weight
+    // fragments of k step q % 2, which the next tile's reads may only replace after the last tail group that
+    // uses them (k step 0: group 2, k step 1: group 3).
     constexpr int kTail = kFa;
-    constexpr int kFbStart0 = NBLK >= kTail ? 0 : kTail / 2 - 1;  // start() call that reads the weights of k step 0
-    // barrier B comes after this many pairs of the tile: the burst of reads at its start has returned by
+    static_assert(kTail == 4 && kKSteps == 2, "the start of a tile is written out for a tail of four groups");
+    // barrier B comes after this many MFMA groups of the tile: the burst of reads at its start has returned by
     // then, so the wait in front of the barrier costs nothing
-    constexpr int kPairsBeforeB = NF - kTail < 6 ? NF - kTail : 6;
-    // The copies of a tile are spread over the MFMA pairs between its barriers instead of following the
+    constexpr int kGroupsBeforeB = NF - kTail < 6 ? NF - kTail : 6;
+    // The copies of a tile are spread over the MFMA groups between its barriers instead of following the
     // barrier in one burst: a copy cannot issue while the L1's queue of pending requests is full, a wave
     // stuck at a copy issues no MFMAs, and a burst of four or five copies from each of the eight waves is
     // several queues long - while the queue, once the burst is in, drains with nothing behind it until the
-    // next barrier.  One copy every other pair keeps the queue fed at the rate it empties and costs a wave
+    // next barrier.  One copy every other group keeps the queue fed at the rate it empties and costs a wave
     // a few lines' worth of waiting at a time, which the MFMAs in flight cover.
-    constexpr int kSlotsA = LIVE > 0 ? kTail + kPairsBeforeB : 0;  // tail pairs + pairs between barrier A and barrier B
-    constexpr int kSlotsB = NF - kTail - kPairsBeforeB;            // pairs between barrier B and the next barrier A
+    constexpr int kSlotsA = LIVE > 0 ? kTail + kGroupsBeforeB : 0;  // tail groups + groups between barrier A and barrier B
+    constexpr int kSlotsB = NF - kTail - kGroupsBeforeB;            // groups between barrier B and the next barrier A
     auto tile = [&](auto stage_c, int kx, int kw, bool tail, bool switch_x, bool switch_w) {
       constexpr int STAGE = decltype(stage_c)::value;
       if (switch_x) set_x_sources(nxt);
@@ -397,35 +396,35 @@ __global__ __launch_bounds__(2 * WN * kWave) void grouped_matmul_persistent_kern
       };
       if constexpr (kSlotsA == 0) copy_x(kx, STAGE ^ 1);
       if constexpr (LIVE > 0) {
-        auto start = [&](auto q_c) {  // tail pair q of the previous tile, then the reads that reuse its registers
+        auto start = [&](auto q_c) {  // tail group q of the previous tile, then the reads that reuse its registers
           constexpr int Q = decltype(q_c)::value;
           if (tail) mma(std::integral_constant<int, NF - kTail + Q>{});
           x_copies_of_slot(Q);
           read_fa(q_c, stage_c);
           __builtin_amdgcn_sched_barrier(0);  // the counted wait in front of barrier B relies on this order
           if constexpr (Q == 2) read_fb(std::integral_constant<int, 0>{}, stage_c);
-          if constexpr (Q == kTail - 1) read_fb(std::integral_constant<int, 1>{}, stage_c);
+          if constexpr (Q == 3) read_fb(std::integral_constant<int, 1>{}, stage_c);
           __builtin_amdgcn_sched_barrier(0);
         };
         start(std::integral_constant<int, 0>{});
         start(std::integral_constant<int, 1>{});
         start(std::integral_constant<int, 2>{});
         start(std::integral_constant<int, 3>{});
-        pairs(pairs, std::integral_constant<int, 0>{}, std::integral_constant<int, kPairsBeforeB>{}, stage_c,
+        groups(groups, std::integral_constant<int, 0>{}, std::integral_constant<int, kGroupsBeforeB>{}, stage_c,
               [&](auto n_c) { x_copies_of_slot(kTail + decltype(n_c)::value); });
       }
       // all own weight fragments of this tile are in registers (LDS serves a wave's reads in order, and only
-      // the kPairsBeforeB refills of the activation ring were issued after the last of them) ...
+      // the kGroupsBeforeB refills of the activation ring were issued after the last of them) ...
       __builtin_amdgcn_sched_barrier(0);
-      __builtin_amdgcn_s_waitcnt(0xc07f | ((LIVE > 0 ? kPairsBeforeB : 0) << 8));  // lgkmcnt only
+      __builtin_amdgcn_s_waitcnt(0xc07f | ((LIVE > 0 ? kGroupsBeforeB : 0) << 8));  // lgkmcnt only
       fence();
       __builtin_amdgcn_s_barrier();  // ... and so are everybody else's: barrier B
       fence();
       if (switch_w) set_w_sources(nxt);
       if constexpr (kSlotsB == 0) copy_w(kw, STAGE);
       if constexpr (LIVE > 0)
-        pairs(pairs, std::integral_constant<int, kPairsBeforeB>{}, std::integral_constant<int, NF - kTail>{}, stage_c,
-              [&](auto n_c) { w_copies_of_slot(decltype(n_c)::value - kPairsBeforeB); });
+        groups(groups, std::integral_constant<int, kGroupsBeforeB>{}, std::integral_constant<int, NF - kTail>{}, stage_c,
+              [&](auto n_c) { w_copies_of_slot(decltype(n_c)::value - kGroupsBeforeB); });
       // own copies of the next tile (all but the weight copies just issued) and all own fragment reads of
       // this tile are complete ...
       __builtin_amdgcn_sched_barrier(0);
